@@ -1,0 +1,291 @@
+"""CPU oracle for the fused normalization path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg may import
+this module; the shipped operators never do.
+
+It restates, in plain PyTorch CPU ops, the eager formulas the reference uses
+when its fused kernels are off -- the behaviour the fused kernels must match:
+
+  * RMSNorm  -- teletron/models/dit/dit_fusedlayers.py:360-370
+        out = (x.float() * rsqrt(x.float().pow(2).mean(-1, keepdim=True) + eps)).type_as(x) * weight
+  * AdaLN    -- teletron/models/dit/dit_fusedlayers.py:198,223 (and :251,271)
+        out = LayerNorm(C, elementwise_affine=False, eps)(x) * (1 + scale[:, None]) + shift[:, None]
+
+Three layers of the same math live here, each one a check on the others:
+
+  eager_*     the formulas above, verbatim in behaviour, differentiated by
+              torch.autograd (this is what "parity with eager" means);
+  staged_*    the same arithmetic written out by hand with every rounding
+              point explicit (the order a fused kernel has to follow);
+  truth_*     float64 closed forms with no intermediate rounding.
+
+What pins the arithmetic (see tests/test_oracle.py): library routines
+(F.rms_norm, F.layer_norm with weight=1+scale, bias=shift), closed forms on
+constant / unit-weight rows, scale and affine invariances, the orthogonality
+invariants of the backward (sum_c dx = 0, sum_c dx*xhat = 0), brute-force
+float64 loops on tiny inputs, torch.autograd.gradcheck, and an independent
+scalar C restatement (oracle/norm_oracle_c.c) that models the bf16 rounding
+points bit by bit.  The reference's own tests hold no vectors for this path.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+EPS = 1e-6  # teletron/models/hunyuanvideo/model.py:109 (layernorm_epsilon)
+
+
+# --------------------------------------------------------------------------
+# eager: the reference's fallback formulas, differentiated by autograd
+# --------------------------------------------------------------------------
+
+def eager_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = EPS) -> torch.Tensor:
+    """dit_fusedlayers.py:360-361,369-370."""
+    xf = x.float()
+    normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return normed.type_as(x) * weight
+
+
+def eager_adaln(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor,
+                eps: float = EPS) -> torch.Tensor:
+    """dit_fusedlayers.py:198 + :223.  x [B,S,C]; scale, shift [B,C]."""
+    xn = F.layer_norm(x, (x.shape[-1],), None, None, eps)
+    return xn * (1 + scale[:, None]) + shift[:, None]
+
+
+def eager_rmsnorm_fwd_bwd(x, weight, grad, eps: float = EPS):
+    """Returns (out, dx, dweight) exactly as autograd produces them."""
+    x = x.detach().clone().requires_grad_(True)
+    weight = weight.detach().clone().requires_grad_(True)
+    out = eager_rmsnorm(x, weight, eps)
+    out.backward(grad)
+    return out.detach(), x.grad, weight.grad
+
+
+def eager_adaln_fwd_bwd(x, scale, shift, grad, eps: float = EPS):
+    """Returns (out, dx, dscale, dshift) exactly as autograd produces them."""
+    x = x.detach().clone().requires_grad_(True)
+    scale = scale.detach().clone().requires_grad_(True)
+    shift = shift.detach().clone().requires_grad_(True)
+    out = eager_adaln(x, scale, shift, eps)
+    out.backward(grad)
+    return out.detach(), x.grad, scale.grad, shift.grad
+
+
+# --------------------------------------------------------------------------
+# staged: every rounding point written out (what a fused kernel must follow)
+# --------------------------------------------------------------------------
+
+def staged_rmsnorm_fwd(x, weight, eps: float = EPS):
+    """Returns (out, rstd[rows] fp32).  Rounding points for low-precision x:
+    y -> dtype(x); y*w -> promoted dtype."""
+    xf = x.float()
+    rstd = torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+    y = (xf * rstd).to(x.dtype)
+    return y * weight, rstd.squeeze(-1)
+
+
+def staged_rmsnorm_bwd(x, weight, rstd, grad):
+    """dx = r*(gy - xhat*mean_c(gy*xhat)), dw = sum_rows round(g*y).
+    gy = g*w is rounded to the promoted dtype first (that is how autograd
+    materialises it); y is the dtype(x)-rounded normalised row."""
+    C = x.shape[-1]
+    xf = x.float()
+    r = rstd.reshape(*x.shape[:-1], 1)
+    xhat = xf * r
+    y = xhat.to(x.dtype)
+    gy = (grad * weight).float()
+    m = (gy * xhat).sum(-1, keepdim=True) / C
+    dx = (r * (gy - xhat * m)).to(x.dtype)
+    prod = grad * y                                   # rounded to the promoted dtype
+    dw = prod.reshape(-1, C).sum(0).to(weight.dtype)  # fp32 accumulation inside sum
+    return dx, dw
+
+
+def staged_adaln_fwd(x, scale, shift, eps: float = EPS):
+    """Returns (out, mean[rows], rstd[rows]).  Rounding points (bf16 case):
+    xn; t = 1+scale; p = xn*t; out = p+shift."""
+    xf = x.float()
+    mean = xf.mean(-1, keepdim=True)
+    var = ((xf - mean) ** 2).mean(-1, keepdim=True)
+    rstd = torch.rsqrt(var + eps)
+    xn = ((xf - mean) * rstd).to(x.dtype)
+    t = 1 + scale[:, None]
+    p = xn * t
+    out = p + shift[:, None]
+    return out, mean.squeeze(-1), rstd.squeeze(-1)
+
+
+def staged_adaln_bwd(x, scale, mean, rstd, grad):
+    """dshift = sum_s g; dscale = sum_s round(g*xn); gx = round(g*t);
+    dx = r*(gx - mean_c(gx) - xhat*mean_c(gx*xhat))."""
+    B, S, C = x.shape
+    xf = x.float()
+    mu = mean.reshape(B, S, 1)
+    r = rstd.reshape(B, S, 1)
+    xhat = (xf - mu) * r
+    xn = xhat.to(x.dtype)
+    t = 1 + scale[:, None]
+    gx = (grad * t).float()
+    m1 = gx.sum(-1, keepdim=True) / C
+    m2 = (gx * xhat).sum(-1, keepdim=True) / C
+    dx = (r * (gx - m1 - xhat * m2)).to(x.dtype)
+    dshift = grad.sum(1).to(scale.dtype)
+    dscale = (grad * xn).sum(1).to(scale.dtype)
+    return dx, dscale, dshift
+
+
+# --------------------------------------------------------------------------
+# truth: float64 closed forms, no intermediate rounding
+# --------------------------------------------------------------------------
+
+def truth_rmsnorm_fwd_bwd(x, weight, grad, eps: float = EPS):
+    C = x.shape[-1]
+    xd, wd, gd = x.double(), weight.double(), grad.double()
+    r = 1.0 / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps)
+    xhat = xd * r
+    out = xhat * wd
+    gy = gd * wd
+    dx = r * (gy - xhat * (gy * xhat).sum(-1, keepdim=True) / C)
+    dw = (gd * xhat).reshape(-1, C).sum(0)
+    return out, dx, dw
+
+
+def truth_adaln_fwd_bwd(x, scale, shift, grad, eps: float = EPS):
+    B, S, C = x.shape
+    xd, sd, hd, gd = x.double(), scale.double(), shift.double(), grad.double()
+    mu = xd.mean(-1, keepdim=True)
+    var = ((xd - mu) ** 2).mean(-1, keepdim=True)
+    r = 1.0 / torch.sqrt(var + eps)
+    xhat = (xd - mu) * r
+    t = 1 + sd[:, None]
+    out = xhat * t + hd[:, None]
+    gx = gd * t
+    dx = r * (gx - gx.mean(-1, keepdim=True) - xhat * (gx * xhat).mean(-1, keepdim=True))
+    return out, dx, (gd * xhat).sum(1), gd.sum(1)
+
+
+# --------------------------------------------------------------------------
+# comparators
+# --------------------------------------------------------------------------
+
+def bf16_ordinal(t: torch.Tensor) -> torch.Tensor:
+    """Monotone integer index of each bf16 value (adjacent values differ by 1;
+    +0 and -0 share index 0)."""
+    assert t.dtype == torch.bfloat16
+    bits = t.contiguous().view(torch.int16).to(torch.int32)
+    return torch.where(bits >= 0, bits, -(bits & 0x7FFF))
+
+
+def bf16_ulp_distance(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    return (bf16_ordinal(a) - bf16_ordinal(b)).abs()
+
+
+@dataclass
+class UlpReport:
+    n: int
+    n_exact: int
+    n_gt1: int          # > 1 ulp and not excused by the cancellation guard
+    n_excused: int      # > 1 ulp but inside the cancellation guard
+    max_ulp: int
+
+    @property
+    def frac_exact(self) -> float:
+        return self.n_exact / max(self.n, 1)
+
+
+def compare_bf16_ulp(got: torch.Tensor, want: torch.Tensor,
+                     cancel_scale: Optional[torch.Tensor] = None) -> UlpReport:
+    """Element-wise bf16 ulp comparison.
+
+    `cancel_scale`, when given, is the magnitude of the larger operand of the
+    final addition (max(|p|, |shift|) for AdaLN).  Two implementations that sum
+    a row in different orders can differ by one ulp in the normalised value xn
+    (a relative step of up to 2^-7); that step is multiplied by 1+scale,
+    re-rounded into p, and then p+shift may cancel, so the result's own ulp can
+    be far finer than the step.  An element more than 1 ulp off is excused iff
+    |got-want| <= 2^-6 * cancel_scale (one relative bf16 step of the operand
+    plus its re-rounding); callers also bound how many elements are excused.
+    """
+    got, want = got.cpu(), want.cpu()
+    d = bf16_ulp_distance(got, want)
+    nan_both = torch.isnan(got) & torch.isnan(want)
+    d = torch.where(nan_both, torch.zeros_like(d), d)
+    bad = d > 1
+    excused = torch.zeros_like(bad)
+    if cancel_scale is not None and bad.any():
+        diff = (got.float() - want.float()).abs()
+        excused = bad & (diff <= cancel_scale.float().cpu() * 2.0 ** -6)
+    return UlpReport(n=d.numel(), n_exact=int((d == 0).sum()),
+                     n_gt1=int((bad & ~excused).sum()), n_excused=int(excused.sum()),
+                     max_ulp=int(d.max()) if d.numel() else 0)
+
+
+def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float) -> float:
+    """Fraction of elements with |got-want| > atol + rtol*|want| (allclose's rule)."""
+    g, w = got.double().cpu(), want.double().cpu()
+    if g.numel() == 0:
+        return 0.0
+    return float(((g - w).abs() > atol + rtol * w.abs()).double().mean())
+
+
+# --------------------------------------------------------------------------
+# seeded inputs for the benchmark configurations
+# --------------------------------------------------------------------------
+
+def _gen(seed: int) -> torch.Generator:
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def make_rmsnorm_inputs(lead_shape: Tuple[int, ...], cols: int, dtype: torch.dtype,
+                        seed: int = 0, sigma: float = 1.0) -> Dict[str, torch.Tensor]:
+    """x ~ N(0, sigma), weight ~ N(1, 0.02), upstream grad ~ N(0, 1)."""
+    g = _gen(seed)
+    x = (sigma * torch.randn(*lead_shape, cols, generator=g)).to(dtype)
+    w = (1 + 0.02 * torch.randn(cols, generator=g)).to(dtype)
+    grad = torch.randn(*lead_shape, cols, generator=g).to(dtype)
+    return {"x": x, "weight": w, "grad": grad}
+
+
+def make_adaln_inputs(batch: int, seq: int, cols: int, dtype: torch.dtype,
+                      seed: int = 0, sigma: float = 1.0) -> Dict[str, torch.Tensor]:
+    """x ~ N(0, sigma); per-sample scale, shift ~ N(0, 0.1); grad ~ N(0, 1)."""
+    g = _gen(seed)
+    x = (sigma * torch.randn(batch, seq, cols, generator=g)).to(dtype)
+    scale = (0.1 * torch.randn(batch, cols, generator=g)).to(dtype)
+    shift = (0.1 * torch.randn(batch, cols, generator=g)).to(dtype)
+    grad = torch.randn(batch, seq, cols, generator=g).to(dtype)
+    return {"x": x, "scale": scale, "shift": shift, "grad": grad}
+
+
+CONFIGS = {
+    # name: (op, kwargs) -- the five workloads of the benchmark definition
+    "cfg1_rms_fp32": ("rmsnorm", dict(lead_shape=(2, 4096), cols=3072, dtype=torch.float32)),
+    "cfg2_qk_rms_bf16": ("rmsnorm", dict(lead_shape=(1, 29700, 24), cols=128, dtype=torch.bfloat16)),
+    "cfg3_adaln_bf16": ("adaln", dict(batch=1, seq=29700, cols=3072, dtype=torch.bfloat16)),
+    "cfg4_rms_bf16": ("rmsnorm", dict(lead_shape=(1, 118800), cols=3072, dtype=torch.bfloat16)),
+    "cfg4_adaln_bf16": ("adaln", dict(batch=1, seq=118800, cols=3072, dtype=torch.bfloat16)),
+    "cfg5_adaln_bf16": ("adaln", dict(batch=4, seq=11056, cols=3072, dtype=torch.bfloat16, sigma=2.0)),
+}
+
+
+def make_config_inputs(name: str, seed: int = 0, rows_limit: Optional[int] = None):
+    """Seeded inputs for one named configuration.  `rows_limit` shrinks the
+    token dimension (for quick checks) without changing anything else."""
+    op, kw = CONFIGS[name]
+    kw = dict(kw)
+    if op == "rmsnorm":
+        if rows_limit is not None:
+            lead = list(kw["lead_shape"])
+            lead[1] = min(lead[1], rows_limit)
+            kw["lead_shape"] = tuple(lead)
+        return op, make_rmsnorm_inputs(seed=seed, **kw)
+    if rows_limit is not None:
+        kw["seq"] = min(kw["seq"], rows_limit)
+    return op, make_adaln_inputs(seed=seed, **kw)

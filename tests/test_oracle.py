@@ -1,0 +1,289 @@
+"""Pins the CPU oracle: every check here would fail for a plausible mistake
+(dropped eps, sum instead of mean, unbiased variance, scale instead of 1+scale,
+shift sign, scale/shift applied to the wrong sample, a missing rounding point).
+None of them re-types the oracle's own formula."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import c_oracle as Cc
+from oracle import norm_oracle as O
+from tests.golden_util import load_golden
+
+EPS = 1e-6
+
+
+# ------------------------------------------------------------------ RMSNorm
+
+@pytest.mark.parametrize("cols", [128, 3072])
+def test_rmsnorm_matches_library_rms_norm(cols):
+    d = O.make_rmsnorm_inputs((64,), cols, torch.float32, seed=3)
+    got = O.eager_rmsnorm(d["x"], d["weight"], EPS)
+    want = F.rms_norm(d["x"], (cols,), d["weight"], EPS)
+    torch.testing.assert_close(got, want, rtol=2e-6, atol=1e-7)
+    db = O.make_rmsnorm_inputs((64,), cols, torch.bfloat16, seed=3)
+    gotb = O.eager_rmsnorm(db["x"], db["weight"], EPS)
+    wantb = F.rms_norm(db["x"].float(), (cols,), db["weight"].float(), EPS)
+    # eager rounds twice (y, then y*w): at most one bf16 ulp from the single-rounded value
+    assert O.compare_bf16_ulp(gotb, wantb.bfloat16()).n_gt1 == 0
+
+
+def test_rmsnorm_constant_row_closed_form():
+    cols = 128
+    for c in (0.5, -3.0, 1e-3, 0.0):
+        x = torch.full((1, cols), c)
+        w = torch.linspace(0.5, 1.5, cols)
+        want = w * (c / math.sqrt(c * c + EPS))
+        torch.testing.assert_close(O.eager_rmsnorm(x, w, EPS)[0], want, rtol=1e-6, atol=1e-12)
+
+
+def test_rmsnorm_unit_weight_mean_square():
+    x = 3.0 * torch.randn(16, 3072, generator=torch.Generator().manual_seed(1))
+    out = O.eager_rmsnorm(x, torch.ones(3072), EPS).double()
+    ms = (x.double() ** 2).mean(-1)
+    torch.testing.assert_close((out ** 2).mean(-1), ms / (ms + EPS), rtol=1e-5, atol=0)
+
+
+def test_rmsnorm_eps_matters_and_scale_invariance():
+    x = torch.randn(8, 128, generator=torch.Generator().manual_seed(2))
+    w = torch.ones(128)
+    # eps -> 0: f(a x) = f(x)
+    torch.testing.assert_close(O.eager_rmsnorm(7.0 * x, w, 0.0), O.eager_rmsnorm(x, w, 0.0),
+                               rtol=1e-6, atol=1e-7)
+    # tiny rows: eps dominates, out ~= x / sqrt(eps)
+    tiny = 1e-6 * x
+    torch.testing.assert_close(O.eager_rmsnorm(tiny, w, EPS),
+                               tiny / torch.sqrt((tiny ** 2).mean(-1, keepdim=True) + EPS),
+                               rtol=1e-5, atol=0)
+    assert (O.eager_rmsnorm(tiny, w, EPS).abs() < 0.01).all()
+
+
+def _brute_rmsnorm(x, w, g, eps):
+    """float64 python loops straight from the definitions; d/dx by the quotient rule."""
+    N, C = x.shape
+    out = [[0.0] * C for _ in range(N)]
+    dx = [[0.0] * C for _ in range(N)]
+    dw = [0.0] * C
+    for n in range(N):
+        ms = sum(float(v) ** 2 for v in x[n]) / C
+        r = 1.0 / math.sqrt(ms + eps)
+        for c in range(C):
+            out[n][c] = float(x[n, c]) * r * float(w[c])
+            dw[c] += float(g[n, c]) * float(x[n, c]) * r
+        # d out[n,k] / d x[n,c] = w_k * (delta_kc * r - x_k * x_c * r^3 / C)
+        for c in range(C):
+            s = 0.0
+            for k in range(C):
+                j = float(w[k]) * ((r if k == c else 0.0) - float(x[n, k]) * float(x[n, c]) * r ** 3 / C)
+                s += float(g[n, k]) * j
+            dx[n][c] = s
+    return (torch.tensor(out, dtype=torch.float64), torch.tensor(dx, dtype=torch.float64),
+            torch.tensor(dw, dtype=torch.float64))
+
+
+def test_rmsnorm_truth_vs_bruteforce_and_autograd():
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 16, generator=gen, dtype=torch.float64)
+    w = 1 + 0.1 * torch.randn(16, generator=gen, dtype=torch.float64)
+    g = torch.randn(3, 16, generator=gen, dtype=torch.float64)
+    bo, bdx, bdw = _brute_rmsnorm(x, w, g, EPS)
+    to, tdx, tdw = O.truth_rmsnorm_fwd_bwd(x, w, g, EPS)
+    for a, b in ((bo, to), (bdx, tdx), (bdw, tdw)):
+        torch.testing.assert_close(a.double(), b, rtol=1e-12, atol=1e-13)
+    eo, edx, edw = O.eager_rmsnorm_fwd_bwd(x, w, g, EPS)  # float64 in, so .float() is the only loss
+    for a, b in ((eo, to), (edx, tdx), (edw, tdw)):
+        torch.testing.assert_close(a.double(), b, rtol=1e-5, atol=1e-6)
+
+
+def test_rmsnorm_gradcheck_on_eager_formula():
+    gen = torch.Generator().manual_seed(6)
+    x = torch.randn(2, 8, generator=gen, dtype=torch.float64, requires_grad=True)
+    w = (1 + 0.1 * torch.randn(8, generator=gen, dtype=torch.float64)).requires_grad_(True)
+
+    def f(x, w):  # the eager formula without the .float() down-cast
+        return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + EPS)) * w
+    assert torch.autograd.gradcheck(f, (x, w), eps=1e-6, atol=1e-6)
+    # and the analytic float64 form agrees with autograd of that same formula
+    g = torch.randn(2, 8, generator=gen, dtype=torch.float64)
+    f(x, w).backward(g)
+    _, tdx, tdw = O.truth_rmsnorm_fwd_bwd(x.detach(), w.detach(), g, EPS)
+    torch.testing.assert_close(x.grad, tdx, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(w.grad, tdw, rtol=1e-10, atol=1e-12)
+
+
+def test_rmsnorm_backward_invariants():
+    d = O.make_rmsnorm_inputs((32,), 3072, torch.float32, seed=7)
+    _, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"], eps=0.0)
+    # with eps = 0 the output is invariant to scaling a row, so x . dx = 0 per row
+    dots = (d["x"].double() * dx.double()).sum(-1)
+    scale = (d["x"].double().abs() * dx.double().abs()).sum(-1)
+    assert (dots.abs() / scale).max() < 1e-5
+    # g = 1  =>  dw = column sums of the normalised rows
+    ones = torch.ones_like(d["x"])
+    out1, _, dw1 = O.eager_rmsnorm_fwd_bwd(d["x"], torch.ones(3072), ones)
+    torch.testing.assert_close(dw1, out1.sum(0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("cols,rows", [(128, 2048), (3072, 96)])
+def test_rmsnorm_staged_and_c_agree_with_eager_bf16(cols, rows):
+    d = O.make_rmsnorm_inputs((rows,), cols, torch.bfloat16, seed=8)
+    out, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    so, sr = O.staged_rmsnorm_fwd(d["x"], d["weight"])
+    assert torch.equal(so.view(torch.int16), out.view(torch.int16))       # rounding points are right
+    co, cr = Cc.rmsnorm_fwd(d["x"], d["weight"], EPS)
+    rep = O.compare_bf16_ulp(co, out)
+    assert rep.n_gt1 == 0 and rep.frac_exact > 0.999                       # only summation order differs
+    torch.testing.assert_close(cr, sr, rtol=3e-7, atol=0)
+    # dropping the intermediate rounding of y would show up here as ~20 % one-ulp differences
+    single = (d["x"].float() * sr[:, None] * d["weight"].float()).bfloat16()
+    assert O.compare_bf16_ulp(single, out).frac_exact < 0.9
+    cdx, cdw = Cc.rmsnorm_bwd(d["x"], d["weight"], cr, d["grad"])
+    sdx, sdw = O.staged_rmsnorm_bwd(d["x"], d["weight"], sr, d["grad"])
+    for got in (cdx, sdx):
+        rep = O.compare_bf16_ulp(got, dx)
+        assert rep.frac_exact > 0.999 and O.frac_outside(got, dx, 1e-2, 1e-3) == 0.0
+    for got in (cdw, sdw):
+        assert O.frac_outside(got, dw, 1e-2, 1e-3) == 0.0
+        assert O.compare_bf16_ulp(got, dw).max_ulp <= 2
+
+
+def test_rmsnorm_c_f32_matches_eager():
+    d = O.make_rmsnorm_inputs((64,), 3072, torch.float32, seed=9)
+    out, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    co, cr = Cc.rmsnorm_fwd(d["x"], d["weight"], EPS)
+    cdx, cdw = Cc.rmsnorm_bwd(d["x"], d["weight"], cr, d["grad"])
+    torch.testing.assert_close(co, out, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(cdx, dx, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(cdw, dw, rtol=1e-5, atol=1e-5)
+
+
+# -------------------------------------------------------------------- AdaLN
+
+def test_adaln_matches_library_layer_norm_affine():
+    d = O.make_adaln_inputs(1, 40, 3072, torch.float32, seed=21)
+    got = O.eager_adaln(d["x"], d["scale"], d["shift"], EPS)
+    want = F.layer_norm(d["x"], (3072,), 1 + d["scale"][0], d["shift"][0], EPS)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_adaln_zero_modulation_moments_and_affine_invariance():
+    gen = torch.Generator().manual_seed(22)
+    x = 2.5 * torch.randn(2, 6, 3072, generator=gen) + 1.0
+    z = torch.zeros(2, 3072)
+    out = O.eager_adaln(x, z, z, EPS).double()
+    var = x.double().var(-1, unbiased=False)
+    assert out.mean(-1).abs().max() < 1e-6
+    torch.testing.assert_close(out.var(-1, unbiased=False), var / (var + EPS), rtol=1e-5, atol=0)
+    # the unbiased estimator would differ by C/(C-1) ~ 3e-4: make sure the check can see that
+    assert ((out.var(-1, unbiased=True) - var / (var + EPS)).abs() > 1e-4).all()
+    # LN(a x + b) = LN(x) for a > 0 (eps negligible against var)
+    torch.testing.assert_close(O.eager_adaln(3.0 * x + 5.0, z, z, 0.0), O.eager_adaln(x, z, z, 0.0),
+                               rtol=1e-4, atol=1e-5)
+
+
+def test_adaln_per_sample_modulation_bruteforce():
+    d = O.make_adaln_inputs(3, 5, 3072, torch.float32, seed=23)
+    got = O.eager_adaln(d["x"], d["scale"], d["shift"], EPS)
+    for b in range(3):
+        xb = d["x"][b].double()
+        mu = xb.mean(-1, keepdim=True)
+        sd = torch.sqrt(((xb - mu) ** 2).mean(-1, keepdim=True) + EPS)
+        want = (xb - mu) / sd * (1 + d["scale"][b].double()) + d["shift"][b].double()
+        torch.testing.assert_close(got[b].double(), want, rtol=1e-5, atol=1e-5)
+    # a sample swapped with its neighbour must be detectable
+    swapped = O.eager_adaln(d["x"], d["scale"].flip(0), d["shift"].flip(0), EPS)
+    assert (swapped[0] - got[0]).abs().max() > 0.05
+
+
+def test_adaln_truth_vs_autograd_fp64_and_invariants():
+    gen = torch.Generator().manual_seed(24)
+    B, S, C = 2, 3, 24
+    x = torch.randn(B, S, C, generator=gen, dtype=torch.float64, requires_grad=True)
+    sc = (0.1 * torch.randn(B, C, generator=gen, dtype=torch.float64)).requires_grad_(True)
+    sh = (0.1 * torch.randn(B, C, generator=gen, dtype=torch.float64)).requires_grad_(True)
+    g = torch.randn(B, S, C, generator=gen, dtype=torch.float64)
+    assert torch.autograd.gradcheck(lambda a, b, c: O.eager_adaln(a, b, c, EPS), (x, sc, sh),
+                                    eps=1e-6, atol=1e-6)
+    out = O.eager_adaln(x, sc, sh, EPS)
+    out.backward(g)
+    to, tdx, tds, tdh = O.truth_adaln_fwd_bwd(x.detach(), sc.detach(), sh.detach(), g, EPS)
+    torch.testing.assert_close(out.detach(), to, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(x.grad, tdx, rtol=1e-9, atol=1e-11)
+    torch.testing.assert_close(sc.grad, tds, rtol=1e-9, atol=1e-11)
+    torch.testing.assert_close(sh.grad, tdh, rtol=1e-9, atol=1e-11)
+    # LayerNorm's backward is orthogonal to the all-ones vector and to xhat
+    xd = x.detach()
+    mu = xd.mean(-1, keepdim=True)
+    xhat = (xd - mu) / torch.sqrt(((xd - mu) ** 2).mean(-1, keepdim=True) + EPS)
+    assert tdx.sum(-1).abs().max() < 1e-10
+    # exact only for eps = 0; with eps = 1e-6 and unit variance the residue is O(eps)
+    assert (tdx * xhat).sum(-1).abs().max() < 1e-4
+
+
+def test_adaln_staged_and_c_agree_with_eager_bf16():
+    d = O.make_adaln_inputs(3, 70, 3072, torch.bfloat16, seed=25)
+    out, dx, ds, dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    so, smu, sr = O.staged_adaln_fwd(d["x"], d["scale"], d["shift"])
+    co, cmu, cr = Cc.adaln_fwd(d["x"], d["scale"], d["shift"], EPS)
+    t = (1 + d["scale"][:, None])
+    for got, mu, r in ((so, smu, sr), (co, cmu, cr)):
+        xn = ((d["x"].float() - mu.view(3, 70, 1)) * r.view(3, 70, 1)).bfloat16()
+        guard = torch.maximum((xn * t).float().abs(), d["shift"][:, None].float().abs().expand_as(xn))
+        rep = O.compare_bf16_ulp(got, out, cancel_scale=guard)
+        assert rep.n_gt1 == 0 and rep.n_excused < 1e-4 * rep.n and rep.frac_exact > 0.999, rep
+    torch.testing.assert_close(cr, sr.reshape(-1), rtol=1e-6, atol=0)
+    torch.testing.assert_close(cmu, smu.reshape(-1), rtol=0, atol=1e-6)
+    # a single final rounding (no intermediate bf16 steps) is visibly different from eager
+    single = ((d["x"].float() - smu.view(3, 70, 1)) * sr.view(3, 70, 1) * (1 + d["scale"].float()[:, None])
+              + d["shift"].float()[:, None]).bfloat16()
+    assert O.compare_bf16_ulp(single, out).frac_exact < 0.95
+    cdx, cds, cdh = Cc.adaln_bwd(d["x"], d["scale"], cmu, cr, d["grad"])
+    sdx, sds, sdh = O.staged_adaln_bwd(d["x"], d["scale"], smu, sr, d["grad"])
+    for gdx, gds, gdh in ((cdx, cds, cdh), (sdx, sds, sdh)):
+        assert O.frac_outside(gdx, dx, 1e-2, 1e-3) < 1e-5
+        assert O.frac_outside(gds, ds, 1e-2, 1e-3) == 0.0
+        assert O.frac_outside(gdh, dh, 1e-2, 1e-3) == 0.0
+    # and against the float64 truth (bf16 rounding noise only)
+    _, tdx, tds, tdh = O.truth_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"], EPS)
+    assert O.frac_outside(cdx, tdx, 2e-2, 2e-2) < 1e-4
+
+
+def test_adaln_c_f32_matches_eager():
+    d = O.make_adaln_inputs(2, 9, 3072, torch.float32, seed=26)
+    out, dx, ds, dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    co, cmu, cr = Cc.adaln_fwd(d["x"], d["scale"], d["shift"], EPS)
+    cdx, cds, cdh = Cc.adaln_bwd(d["x"], d["scale"], cmu, cr, d["grad"])
+    torch.testing.assert_close(co, out, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(cdx, dx, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(cds, ds, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(cdh, dh, rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------ golden vectors
+
+def test_golden_vectors_reproduce():
+    gold = load_golden()
+    assert len(gold) == 7
+    for name, d in gold.items():
+        if name.startswith("rms"):
+            out, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+            got = {"out": out, "dx": dx, "dweight": dw}
+        else:
+            out, dx, ds, dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+            got = {"out": out, "dx": dx, "dscale": ds, "dshift": dh}
+        for k, v in got.items():
+            if d["is_bf16"]:
+                # thread count may change a summation order: allow 1 ulp on a handful of elements
+                rep = O.compare_bf16_ulp(v, d[k])
+                assert rep.frac_exact > 0.995 and O.frac_outside(v, d[k], 1e-2, 1e-3) == 0.0, (name, k, rep)
+            else:
+                torch.testing.assert_close(v, d[k], rtol=1e-5, atol=1e-5)
+
+
+def test_bf16_ulp_comparator():
+    a = torch.tensor([1.0, 1.0, -1.0, 0.0, 2.0 ** -126]).bfloat16()
+    b = torch.tensor([1.0078125, 1.015625, -1.0078125, -0.0, 0.0]).bfloat16()
+    assert O.bf16_ulp_distance(a, b).tolist() == [1, 2, 1, 0, 128]
