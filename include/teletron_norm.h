@@ -1,0 +1,146 @@
+/* teletron_norm.h -- C ABI of the gfx950 fused normalization library
+ * (libteletron_norm.so): fused RMSNorm and fused AdaLayerNorm, forward and
+ * backward, for bf16 and fp32 rows of 128 or 3072 columns.
+ *
+ * This is the seam the reference has between its pybind glue and its kernel
+ * launchers (teletron_op/fused_rmsnorm/include/rmsnorm_kernel.h:5-25 and
+ * teletron_op/fused_adaln/include/adaln_kernel.h:20-45): plain device
+ * pointers and sizes in, nothing returned but a status.  Differences from
+ * those launchers, all additive:
+ *   - every call takes the HIP stream to enqueue on (the reference launches
+ *     on the legacy default stream) and returns a status instead of void;
+ *   - the element type is an argument (the reference is bf16 only);
+ *   - AdaLN takes one scale/shift row PER SAMPLE ([batch, cols]), as the
+ *     eager path does (teletron/models/dit/dit_fusedlayers.py:223); the
+ *     reference kernels read a single row;
+ *   - the backward entry points come in two flavours: the native one works
+ *     from the saved INPUT x and row statistics (forward writes 1 tensor),
+ *     the *_from_out / *_from_xnorm ones work from what the reference's
+ *     Python functions save (forward output / normalised x) so the
+ *     reference's autograd classes run unmodified;
+ *   - scratch memory for the parameter-gradient partial sums is passed in by
+ *     the caller (query the size first); the library never allocates.
+ *
+ * All pointers are device pointers, 16-byte aligned, row-major contiguous.
+ * All calls are asynchronous on `stream` (a hipStream_t passed as void*;
+ * NULL = the null stream).  Nothing here synchronises.
+ */
+#ifndef TELETRON_NORM_H_
+#define TELETRON_NORM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TT_NORM_ABI_VERSION 1
+
+enum tt_norm_status {
+    TT_NORM_OK = 0,
+    TT_NORM_EINVAL = 1,       /* null pointer, non-positive size, rows not divisible by batch */
+    TT_NORM_EUNSUPPORTED = 2, /* cols or dtype the kernels are not built for */
+    TT_NORM_EALIGN = 3,       /* a tensor pointer is not 16-byte aligned */
+    TT_NORM_EWORKSPACE = 4,   /* workspace missing or smaller than *_workspace_bytes() */
+    TT_NORM_EHIP = 5          /* the HIP runtime refused the launch; see tt_norm_last_error() */
+};
+
+enum tt_norm_dtype {
+    TT_NORM_BF16 = 0,
+    TT_NORM_F32 = 1
+};
+
+/* ABI version of the loaded library (TT_NORM_ABI_VERSION at build time). */
+int tt_norm_abi_version(void);
+
+/* Static description of a status code. */
+const char *tt_norm_status_string(int status);
+
+/* Thread-local detail of the last non-OK status returned on this thread. */
+const char *tt_norm_last_error(void);
+
+/* 1 if (cols, dtype) is a shape the kernels are built for, else 0. */
+int tt_norm_supported(int64_t cols, int dtype);
+
+/* ------------------------------------------------------------------ RMSNorm
+ * out = round(round(x * rstd) * weight),  rstd = 1/sqrt(mean_c(x^2) + eps)
+ * (intermediate rounding to the element type as the eager path does,
+ * teletron/models/dit/dit_fusedlayers.py:360-370).
+ */
+
+/* Replaces launch_rms_forward (rmsnorm_kernel.h:5-12, rms_forward.cu:102).
+ * out [rows, cols], rstd [rows] fp32 (the reference's inv_variance). */
+int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight,
+                       int64_t rows, int64_t cols, double eps, int dtype, void *stream);
+
+/* Bytes of scratch tt_rmsnorm_backward* need for this shape. */
+size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+
+/* Native backward from the saved input: dx [rows, cols], dweight [cols].
+ * One pass over dout and x produces dx and per-workgroup partial column sums;
+ * a second small kernel reduces the partials in a fixed order (deterministic).
+ * Covers launch_rms_backward + launch_rms_weight_backward
+ * (rms_backward.cu:91, weight_backward.cu:212). */
+int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x,
+                        const void *weight, const float *rstd,
+                        int64_t rows, int64_t cols, int dtype,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+/* Same contract as the reference's launch_rms_backward (rmsnorm_kernel.h:19-24):
+ * `out` is the saved FORWARD OUTPUT; the normalised row is recovered as
+ * out / weight (weight must be non-zero, as in the reference). */
+int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, const void *out,
+                                 const void *weight, const float *rstd,
+                                 int64_t rows, int64_t cols, int dtype,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* -------------------------------------------------------------------- AdaLN
+ * out = round(round(LN(x) * round(1 + scale[b])) + shift[b]),  LN without affine,
+ * b = row / rows_per_sample  (teletron/models/dit/dit_fusedlayers.py:198,223).
+ * x, out [batch * rows_per_sample, cols]; scale, shift [batch, cols].
+ */
+
+/* Native forward: writes out and the per-row statistics mean, rstd [rows] fp32. */
+int tt_adaln_forward(void *out, float *mean, float *rstd, const void *x,
+                     const void *scale, const void *shift,
+                     int64_t batch, int64_t rows_per_sample, int64_t cols,
+                     double eps, int dtype, void *stream);
+
+/* Replaces launch_adaln_forward (adaln_kernel.h:20-29, adaln_forward.cu:198):
+ * additionally writes x_norm [rows, cols] = round(LN(x)); rstd is the
+ * reference's inv_variance. */
+int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x,
+                           const void *scale, const void *shift,
+                           int64_t batch, int64_t rows_per_sample, int64_t cols,
+                           double eps, int dtype, void *stream);
+
+size_t tt_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample,
+                                         int64_t cols, int dtype);
+
+/* Native backward from the saved input and statistics: dx [rows, cols],
+ * dscale, dshift [batch, cols].  Covers launch_adaln_backward +
+ * launch_adaln_scale_shift_backward (adaln_backward.cu:129,
+ * scale_shift_backward.cu:129) in one pass plus the fixed-order reducer. */
+int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                      const void *scale, const float *mean, const float *rstd,
+                      int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* Same contract as the reference's launch_adaln_backward (adaln_kernel.h:36-45):
+ * works from the saved normalised rows x_norm and rstd. */
+int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const void *dout,
+                                 const void *x_norm, const void *scale, const float *rstd,
+                                 int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------- measurement
+ * Plain streaming copy of `bytes` (multiple of 16) from src to dst with the
+ * same 128-bit access pattern as the kernels: the achievable-bandwidth
+ * yardstick the benchmark prints next to each result. */
+int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TELETRON_NORM_H_ */

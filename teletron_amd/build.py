@@ -1,0 +1,89 @@
+"""Build recipe for the native parts, all compiled for gfx950 and kept in-tree:
+
+  teletron_amd/lib/libteletron_norm.so   HIP kernels + C ABI (include/teletron_norm.h)
+  teletron_amd/ext/fused_rmsnorm*.so     PyTorch extension modules with the reference's
+  teletron_amd/ext/fused_adaln*.so       module names and torch_launch_* signatures
+
+Run `python -m teletron_amd.build` (hipcc cross-compiles; no GPU needed).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+import sysconfig
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIB_DIR = os.path.join(PKG, "lib")
+EXT_DIR = os.path.join(PKG, "ext")
+LIB_PATH = os.path.join(LIB_DIR, "libteletron_norm.so")
+
+HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+ARCH = "gfx950"
+# -packed-fp32-ops off: scalar fp32 VALU only (packed fp32 forms are not trusted on this fleet)
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip"]
+EXT_MODULES = {"fused_rmsnorm": "fused_rmsnorm_ext.cpp", "fused_adaln": "fused_adaln_ext.cpp"}
+
+
+def _run(cmd, cwd=None):
+    proc = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # hipcc's host pass says it does not know the packed-fp32 feature; that is expected
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_kernels(verbose: bool = True) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [HIPCC, *HIP_FLAGS, "-shared", "-o", LIB_PATH] + KERNEL_SOURCES
+    out = _run(cmd, cwd=CSRC)
+    if verbose:
+        print("built", os.path.relpath(LIB_PATH, ROOT), out.strip())
+    return LIB_PATH
+
+
+def ext_path(name: str) -> str:
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    return os.path.join(EXT_DIR, name + suffix)
+
+
+def build_extensions(verbose: bool = True):
+    """The two PyTorch extension modules: host-only C++ (argument checks, current
+    stream, workspace from the caching allocator) linked against the C ABI."""
+    from torch.utils import cpp_extension as ce
+    import torch
+
+    os.makedirs(EXT_DIR, exist_ok=True)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = [f"-I{p}" for p in ce.include_paths()]
+    inc += ["-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(ROOT, "include"),
+            "-I/opt/rocm/include"]
+    paths = []
+    for name, src in EXT_MODULES.items():
+        out = ext_path(name)
+        cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+               f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+               *inc, os.path.join(CSRC, src), "-o", out,
+               f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-ltorch_python",
+               f"-L{LIB_DIR}", "-lteletron_norm",
+               "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{torch_lib}"]
+        log = _run(cmd)
+        if verbose:
+            print("built", os.path.relpath(out, ROOT), log.strip())
+        paths.append(out)
+    return paths
+
+
+def build_all(verbose: bool = True):
+    build_kernels(verbose)
+    build_extensions(verbose)
+
+
+if __name__ == "__main__":
+    build_all()

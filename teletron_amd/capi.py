@@ -1,0 +1,177 @@
+"""ctypes view of the C ABI in include/teletron_norm.h, taking torch tensors.
+
+Thin on purpose: it forwards device pointers, sizes and the current HIP stream
+to libteletron_norm.so and raises on a non-zero status.  There is no fallback:
+if the library is not built, loading fails with instructions to build it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libteletron_norm.so")
+
+BF16, F32 = 0, 1
+_DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
+
+EXPORTS = (
+    "tt_norm_abi_version", "tt_norm_status_string", "tt_norm_last_error", "tt_norm_supported",
+    "tt_rmsnorm_forward", "tt_rmsnorm_backward_workspace_bytes", "tt_rmsnorm_backward",
+    "tt_rmsnorm_backward_from_out",
+    "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
+    "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
+)
+
+
+class NormError(RuntimeError):
+    def __init__(self, status: int, what: str, detail: str):
+        super().__init__(f"{what}: status {status} ({detail})")
+        self.status = status
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(f"{_LIB_PATH} is not built; run `python -m teletron_amd.build`")
+        L = ctypes.CDLL(_LIB_PATH)
+        i64, vp, dbl, ci, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_double, ctypes.c_int, ctypes.c_size_t
+        L.tt_norm_abi_version.restype = ci
+        L.tt_norm_status_string.restype = ctypes.c_char_p
+        L.tt_norm_status_string.argtypes = [ci]
+        L.tt_norm_last_error.restype = ctypes.c_char_p
+        L.tt_norm_supported.argtypes = [i64, ci]
+        L.tt_rmsnorm_forward.argtypes = [vp, vp, vp, vp, i64, i64, dbl, ci, vp]
+        L.tt_rmsnorm_backward_workspace_bytes.restype = sz
+        L.tt_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64, ci]
+        L.tt_rmsnorm_backward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp, sz, vp]
+        L.tt_rmsnorm_backward_from_out.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp, sz, vp]
+        L.tt_adaln_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
+        L.tt_adaln_forward_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
+        L.tt_adaln_backward_workspace_bytes.restype = sz
+        L.tt_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
+        L.tt_adaln_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
+        L.tt_adaln_backward_from_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
+        L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
+        _lib = L
+    return _lib
+
+
+def _check(status: int, what: str):
+    if status != 0:
+        L = lib()
+        raise NormError(status, what, (L.tt_norm_last_error() or L.tt_norm_status_string(status)).decode())
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {t.dtype}")
+    return _DTYPES[t.dtype]
+
+
+def _dense_gpu(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise ValueError("tensor must live on the GPU")
+        if not t.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+
+
+def _workspace(nbytes: int, like: torch.Tensor) -> torch.Tensor:
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=like.device)
+
+
+def rmsnorm_forward(x, weight, eps: float, out=None, rstd=None):
+    _dense_gpu(x, weight)
+    cols = weight.numel()
+    rows = x.numel() // cols
+    out = torch.empty_like(x) if out is None else out
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device) if rstd is None else rstd
+    with torch.cuda.device(x.device):
+        _check(lib().tt_rmsnorm_forward(_p(out), _p(rstd), _p(x), _p(weight), rows, cols, eps, _dt(x),
+                                        _stream(x)), "tt_rmsnorm_forward")
+    return out, rstd
+
+
+def rmsnorm_backward(dout, x, weight, rstd, from_out: bool = False, dx=None, dweight=None):
+    _dense_gpu(dout, x, weight, rstd)
+    cols = weight.numel()
+    rows = x.numel() // cols
+    dx = torch.empty_like(x) if dx is None else dx
+    dweight = torch.empty_like(weight) if dweight is None else dweight
+    with torch.cuda.device(x.device):
+        L = lib()
+        n = L.tt_rmsnorm_backward_workspace_bytes(rows, cols, _dt(x))
+        ws = _workspace(n, x)
+        fn = L.tt_rmsnorm_backward_from_out if from_out else L.tt_rmsnorm_backward
+        _check(fn(_p(dx), _p(dweight), _p(dout), _p(x), _p(weight), _p(rstd), rows, cols, _dt(x),
+                  _p(ws), n, _stream(x)), fn.__name__)
+    return dx, dweight
+
+
+def adaln_forward(x, scale, shift, eps: float, want_xnorm: bool = False):
+    """x [B, S, C] (or [rows, C] with scale [1, C]); returns (out, mean, rstd) or
+    (out, x_norm, rstd) when want_xnorm."""
+    _dense_gpu(x, scale, shift)
+    cols = x.shape[-1]
+    batch = scale.numel() // cols
+    rows = x.numel() // cols
+    if rows % batch:
+        raise ValueError("rows not divisible by batch")
+    out = torch.empty_like(x)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        if want_xnorm:
+            xn = torch.empty_like(x)
+            _check(lib().tt_adaln_forward_xnorm(_p(out), _p(xn), _p(rstd), _p(x), _p(scale), _p(shift), batch,
+                                                rows // batch, cols, eps, _dt(x), _stream(x)),
+                   "tt_adaln_forward_xnorm")
+            return out, xn, rstd
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        _check(lib().tt_adaln_forward(_p(out), _p(mean), _p(rstd), _p(x), _p(scale), _p(shift), batch,
+                                      rows // batch, cols, eps, _dt(x), _stream(x)), "tt_adaln_forward")
+    return out, mean, rstd
+
+
+def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False):
+    _dense_gpu(dout, x, scale, rstd)
+    cols = x.shape[-1]
+    batch = scale.numel() // cols
+    rows = x.numel() // cols
+    dx = torch.empty_like(x)
+    dscale = torch.empty_like(scale)
+    dshift = torch.empty_like(scale)
+    with torch.cuda.device(x.device):
+        L = lib()
+        n = L.tt_adaln_backward_workspace_bytes(batch, rows // batch, cols, _dt(x))
+        ws = _workspace(n, x)
+        if from_xnorm:
+            _check(L.tt_adaln_backward_from_xnorm(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(x), _p(scale),
+                                                  _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n,
+                                                  _stream(x)), "tt_adaln_backward_from_xnorm")
+        else:
+            _check(L.tt_adaln_backward(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(x), _p(scale), _p(mean),
+                                       _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n, _stream(x)),
+                   "tt_adaln_backward")
+    return dx, dscale, dshift
+
+
+def stream_copy(dst: torch.Tensor, src: torch.Tensor):
+    _dense_gpu(dst, src)
+    nbytes = src.numel() * src.element_size()
+    with torch.cuda.device(src.device):
+        _check(lib().tt_norm_stream_copy(_p(dst), _p(src), nbytes, _stream(src)), "tt_norm_stream_copy")

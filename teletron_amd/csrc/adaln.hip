@@ -1,0 +1,379 @@
+// Fused AdaLayerNorm for gfx950: LayerNorm without affine, then per-sample
+// modulation  out = LN(x) * (1 + scale[b]) + shift[b];  forward, and a
+// single-pass backward producing dx plus per-workgroup partial column sums
+// for dscale and dshift.
+//
+// Math (rounding points follow the eager graph of
+// teletron/models/dit/dit_fusedlayers.py:198,223; "rnd" = round to the element
+// type, identity for fp32):
+//   forward   mu = mean_c(x); r = 1/sqrt(mean_c((x-mu)^2) + eps)
+//             xn = rnd((x-mu)*r); t = rnd(1+scale[b]); out = rnd(rnd(xn*t) + shift[b])
+//   backward  gx = rnd(g*t); xhat = (x-mu)*r
+//             dx = rnd(r*(gx - mean_c(gx) - xhat*mean_c(gx*xhat)))
+//             dshift[b,c] = sum_s g;  dscale[b,c] = sum_s rnd(g * rnd(xhat))
+// The variance is taken about the mean over the row held in registers (two
+// passes over registers, one over memory).  HBM traffic per row: forward reads
+// x and writes out (+8 B of statistics); backward reads g and x, writes dx.
+#include "norm_device.h"
+#include "norm_host.h"
+
+namespace ttn {
+
+// Loads this sample's modulation row and returns t = rnd(1 + scale) packed in
+// the element type.
+template <typename T, int C>
+__device__ __forceinline__ void load_one_plus_scale(u32x4 *tr, const T *__restrict__ scale_row, int l) {
+    using G = RowGeom<T, C>;
+    using E = Elem<T>;
+#pragma unroll
+    for (int k = 0; k < G::CHUNKS; ++k) {
+        float v[G::VEC];
+        E::unpack(load16(reinterpret_cast<const u32x4 *>(scale_row) + k * G::LANES + l), v);
+#pragma unroll
+        for (int j = 0; j < G::VEC; ++j) v[j] = 1.0f + v[j];
+        tr[k] = E::pack(v);
+    }
+}
+
+template <typename T, int C, bool WRITE_XNORM>
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2) void adaln_fwd_kernel(
+    T *__restrict__ out, T *__restrict__ xnorm, float *__restrict__ mean, float *__restrict__ rstd,
+    const T *__restrict__ x, const T *__restrict__ scale, const T *__restrict__ shift,
+    int64_t rows_per_sample, int blocks_per_sample, float eps) {
+    using G = RowGeom<T, C>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const int64_t b = blockIdx.x / blocks_per_sample;
+    const int slot = blockIdx.x % blocks_per_sample;
+
+    u32x4 tr[CHUNKS], hr[CHUNKS];
+    load_one_plus_scale<T, C>(tr, scale + b * C, l);
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) hr[k] = load16(reinterpret_cast<const u32x4 *>(shift + b * C) + k * LANES + l);
+
+    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
+    for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(tr);
+        keep_packed(hr);
+        const int64_t rs = grp * RPW + sub;  // row inside the sample
+        const bool ok = rs < rows_per_sample;
+        const int64_t row = b * rows_per_sample + rs;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(x + row * C) + l;
+        u32x4 xr[CHUNKS];
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += v[j];
+        }
+        const float mu = group_sum<LANES>(s) / (float)C;
+        float q = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float d = v[j] - mu;
+                q = fmaf(d, d, q);
+            }
+        }
+        const float r = 1.0f / sqrtf(group_sum<LANES>(q) / (float)C + eps);
+        if (ok && l == 0) {
+            if (mean) mean[row] = mu;
+            rstd[row] = r;
+        }
+
+        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+        u32x4 *pn = WRITE_XNORM ? reinterpret_cast<u32x4 *>(xnorm + row * C) + l : nullptr;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC], tv[VEC], hv[VEC];
+            E::unpack(xr[k], v);
+            E::unpack(tr[k], tv);
+            E::unpack(hr[k], hv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = (v[j] - mu) * r;
+            if constexpr (WRITE_XNORM) {
+                const u32x4 xn = E::pack(v);
+                if (ok) store16_stream(pn + k * LANES, xn);
+                E::unpack(xn, v);
+            } else {
+                E::round(v);  // xn
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= tv[j];
+            E::round(v);  // xn * (1 + scale)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += hv[j];
+            if (ok) store16_stream(po + k * LANES, E::pack(v));
+        }
+    }
+}
+
+// FROM_XNORM = false: xin is the saved input x, statistics mean/rstd.
+// FROM_XNORM = true : xin is the saved normalised row rnd(LN(x)); only rstd is used.
+template <typename T, int C, bool FROM_XNORM>
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void adaln_bwd_kernel(
+    T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
+    const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
+    const float *__restrict__ rstd, int64_t rows_per_sample, int blocks_per_sample) {
+    using G = RowGeom<T, C>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    __shared__ float lds[2 * C];
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const int64_t b = blockIdx.x / blocks_per_sample;
+    const int slot = blockIdx.x % blocks_per_sample;
+
+    u32x4 tr[CHUNKS];
+    load_one_plus_scale<T, C>(tr, scale + b * C, l);
+
+    float acc[2][CHUNKS][VEC];  // [0] = dscale, [1] = dshift
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[s][k][j] = 0.0f;
+
+    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
+    for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(tr);
+        const int64_t rs = grp * RPW + sub;
+        const bool ok = rs < rows_per_sample;
+        const int64_t row = b * rows_per_sample + rs;
+        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + row * C) + l;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + row * C) + l;
+        u32x4 gr[CHUNKS], xr[CHUNKS];
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            gr[k] = ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+            xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        }
+        const float r = ok ? rstd[row] : 0.0f;
+        const float mu = (!FROM_XNORM && ok) ? mean[row] : 0.0f;
+
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], xv[VEC], tv[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(xr[k], xv);
+            E::unpack(tr[k], tv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] *= tv[j];
+            E::round(gv);  // gx materialised in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xh = FROM_XNORM ? xv[j] : (xv[j] - mu) * r;
+                s1 += gv[j];
+                s2 = fmaf(gv[j], xh, s2);
+            }
+        }
+        const float m1 = group_sum<LANES>(s1) / (float)C;
+        const float m2 = group_sum<LANES>(s2) / (float)C;
+        const float k0 = -(r * m1), k1 = -(r * m2);  // dx = r*gx + xhat*k1 + k0
+        // Pass 2 re-derives gx and xhat from the packed registers instead of keeping
+        // them live across the reductions (registers buy occupancy here).
+        keep_packed(gr);
+        keep_packed(xr);
+
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], gx[VEC], xv[VEC], tv[VEC], o[VEC], xn[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(xr[k], xv);
+            E::unpack(tr[k], tv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gx[j] = gv[j] * tv[j];
+            E::round(gx);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xh = FROM_XNORM ? xv[j] : (xv[j] - mu) * r;
+                o[j] = fmaf(r, gx[j], fmaf(xh, k1, k0));
+                xn[j] = xh;
+                acc[1][k][j] += gv[j];
+            }
+            if (ok) store16_stream(pd + k * LANES, E::pack(o));
+            if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
+            E::round(xn);  // g*xn materialised in the element type before the column sum
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[0][k][j] += xn[j];
+        }
+    }
+    flush_column_partials<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds);
+}
+
+template <typename T, int C>
+struct AdalnTune {
+    static constexpr int kFwdBlocksPerCu = 8;
+    static constexpr int kBwdBlocksPerCu = 2;
+};
+
+struct AdalnArgs {
+    int64_t batch, rows_per_sample;
+    double eps;
+    hipStream_t stream;
+};
+
+template <typename T, int C, bool WRITE_XNORM>
+static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, const void *x,
+                           const void *scale, const void *shift, const AdalnArgs &a) {
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const RowPlan p = make_row_plan(a.batch, a.rows_per_sample, RowGeom<T, C>::RPW,
+                                    AdalnTune<T, C>::kFwdBlocksPerCu, cus);
+    if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln forward: grid too large");
+    adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+        (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
+        a.rows_per_sample, p.blocks_per_sample, (float)a.eps);
+    return check_launch("adaln forward launch");
+}
+
+template <typename T, int C>
+static RowPlan adaln_backward_plan(int64_t batch, int64_t rows_per_sample, int cus) {
+    return make_row_plan(batch, rows_per_sample, RowGeom<T, C>::RPW, AdalnTune<T, C>::kBwdBlocksPerCu, cus);
+}
+
+template <typename T, int C, bool FROM_XNORM>
+static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g, const void *xin,
+                            const void *scale, const float *mean, const float *rstd, int dtype,
+                            void *ws, size_t ws_bytes, const AdalnArgs &a) {
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const RowPlan p = adaln_backward_plan<T, C>(a.batch, a.rows_per_sample, cus);
+    if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln backward: grid too large");
+    const size_t need = (size_t)p.blocks * 2 * C * sizeof(float);
+    if (!ws || ws_bytes < need)
+        return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
+    adaln_bwd_kernel<T, C, FROM_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
+        a.rows_per_sample, p.blocks_per_sample);
+    st = check_launch("adaln backward launch");
+    if (st != TT_NORM_OK) return st;
+    return launch_colreduce(dscale, dshift, (const float *)ws, a.batch, p.blocks_per_sample, C, 2 * C,
+                            dtype, a.stream);
+}
+
+static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                            int dtype, std::initializer_list<const void *> ptrs) {
+    if (batch <= 0 || rows_per_sample <= 0 || cols <= 0)
+        return fail(TT_NORM_EINVAL, "%s: batch=%lld rows_per_sample=%lld cols=%lld", who, (long long)batch,
+                    (long long)rows_per_sample, (long long)cols);
+    if (!tt_norm_supported(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
+                    (long long)cols, dtype);
+    for (const void *p : ptrs) {
+        if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
+        if (!aligned16(p)) return fail(TT_NORM_EALIGN, "%s: pointer %p not 16-byte aligned", who, p);
+    }
+    return TT_NORM_OK;
+}
+
+}  // namespace ttn
+
+using namespace ttn;
+
+#define TTN_DISPATCH(dtype, cols, CALL)                          \
+    do {                                                         \
+        if ((dtype) == TT_NORM_BF16) {                           \
+            if ((cols) == 128) { CALL(bf16_t, 128); }            \
+            else { CALL(bf16_t, 3072); }                         \
+        } else {                                                 \
+            if ((cols) == 128) { CALL(float, 128); }             \
+            else { CALL(float, 3072); }                          \
+        }                                                        \
+    } while (0)
+
+extern "C" {
+
+int tt_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                     const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                     double eps, int dtype, void *stream) {
+    int st = check_adaln_args("tt_adaln_forward", batch, rows_per_sample, cols, dtype, {out, x, scale, shift});
+    if (st != TT_NORM_OK) return st;
+    if (!mean || !rstd) return fail(TT_NORM_EINVAL, "tt_adaln_forward: null mean/rstd");
+    const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
+#define CALL(T, C) return adaln_forward_t<T, C, false>(out, nullptr, mean, rstd, x, scale, shift, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x, const void *scale,
+                           const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                           double eps, int dtype, void *stream) {
+    int st = check_adaln_args("tt_adaln_forward_xnorm", batch, rows_per_sample, cols, dtype,
+                              {out, x_norm, x, scale, shift});
+    if (st != TT_NORM_OK) return st;
+    if (!rstd) return fail(TT_NORM_EINVAL, "tt_adaln_forward_xnorm: null rstd");
+    const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
+#define CALL(T, C) return adaln_forward_t<T, C, true>(out, x_norm, nullptr, rstd, x, scale, shift, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+size_t tt_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
+    if (batch <= 0 || rows_per_sample <= 0 || !tt_norm_supported(cols, dtype)) return 0;
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return 0;
+#define CALL(T, C) \
+    return (size_t)adaln_backward_plan<T, C>(batch, rows_per_sample, cus).blocks * 2 * C * sizeof(float)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                      const void *scale, const float *mean, const float *rstd, int64_t batch,
+                      int64_t rows_per_sample, int64_t cols, int dtype, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+    int st = check_adaln_args("tt_adaln_backward", batch, rows_per_sample, cols, dtype, {dx, dout, x, scale});
+    if (st != TT_NORM_OK) return st;
+    if (!dscale || !dshift || !mean || !rstd)
+        return fail(TT_NORM_EINVAL, "tt_adaln_backward: null dscale/dshift/mean/rstd");
+    const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
+#define CALL(T, C)                                                                                \
+    return adaln_backward_t<T, C, false>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype, workspace, \
+                                         workspace_bytes, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const void *dout,
+                                 const void *x_norm, const void *scale, const float *rstd,
+                                 int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+    int st = check_adaln_args("tt_adaln_backward_from_xnorm", batch, rows_per_sample, cols, dtype,
+                              {dx, dout, x_norm, scale});
+    if (st != TT_NORM_OK) return st;
+    if (!dscale || !dshift || !rstd)
+        return fail(TT_NORM_EINVAL, "tt_adaln_backward_from_xnorm: null dscale/dshift/rstd");
+    const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
+#define CALL(T, C)                                                                                 \
+    return adaln_backward_t<T, C, true>(dx, dscale, dshift, dout, x_norm, scale, nullptr, rstd, dtype, \
+                                        workspace, workspace_bytes, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+}  // extern "C"

@@ -1,0 +1,210 @@
+// Device-side building blocks shared by the gfx950 normalization kernels:
+// 128-bit row access, bf16 <-> fp32 packing with the hardware RNE convert,
+// wave64 DPP reductions, and the row -> lane geometry.
+//
+// Geometry.  A row of C elements is owned by LANES lanes of one wavefront;
+// every lane moves 16 bytes (VEC elements) per access and a row takes CHUNKS
+// accesses per lane, so each access of a wavefront is one contiguous,
+// fully-coalesced 1 KiB (LANES = 64) segment:
+//     column(chunk k, lane l, element j) = (k * LANES + l) * VEC + j
+//   C = 3072 bf16 : LANES 64, CHUNKS 6  -> one wavefront per row, no LDS
+//   C = 3072 fp32 : LANES 64, CHUNKS 12
+//   C =  128 bf16 : LANES 16, CHUNKS 1  -> four rows per wavefront (one DPP row each)
+//   C =  128 fp32 : LANES 32, CHUNKS 1  -> two rows per wavefront
+// A lane owns the same columns for every row it ever sees, which is what lets
+// the backward kernels keep parameter-gradient partial sums in registers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttn {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// Storage-only tag for bf16 elements (arithmetic is always fp32).
+struct bf16_t {
+    uint16_t bits;
+};
+
+constexpr int kWaveSize = 64;
+constexpr int kRowWaves = 4;  // wavefronts per workgroup of every row kernel
+constexpr int kRowThreads = kRowWaves * kWaveSize;
+
+// Caps a kernel's register use so that at least N wavefronts fit on each SIMD
+// (512 registers per lane per SIMD: N = 4 -> 128 registers, N = 2 -> 256).
+#define TTN_MIN_WAVES_PER_SIMD(N) __attribute__((amdgpu_waves_per_eu(N)))
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Two fp32 -> one dword of two bf16, round-to-nearest-even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    bf16x2_t v;
+    v[0] = (__bf16)lo;
+    v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<bf16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = as_f32(r[i] << 16);
+            v[2 * i + 1] = as_f32(r[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+        return r;
+    }
+    // Round every value to bf16 and back: the eager graph materialises this
+    // tensor in bf16 at this point.
+    static __device__ __forceinline__ void round(float (&v)[8]) {
+        u32x4 r = pack(v);
+        unpack(r, v);
+    }
+};
+
+template <>
+struct Elem<float> {
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&v)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = as_f32(r[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&v)[4]) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = as_u32(v[i]);
+        return r;
+    }
+    static __device__ __forceinline__ void round(float (&)[4]) {}
+};
+
+template <typename T, int C>
+struct RowGeom {
+    static constexpr int VEC = Elem<T>::VEC;
+    static constexpr int LANES = (C / VEC) < kWaveSize ? (C / VEC) : kWaveSize;
+    static constexpr int CHUNKS = C / (VEC * LANES);
+    static constexpr int RPW = kWaveSize / LANES;  // rows per wavefront
+    static_assert(C % (VEC * LANES) == 0, "row must split into whole 16-byte accesses");
+    static_assert(LANES == 16 || LANES == 32 || LANES == 64, "row must fill whole DPP rows");
+};
+
+// Streaming 16-byte accesses.  Activations are touched once per kernel, so
+// they carry the non-temporal hint; parameters use the plain cached forms.
+__device__ __forceinline__ u32x4 load16_stream(const u32x4 *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void store16_stream(u32x4 *p, const u32x4 &v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ u32x4 load16(const u32x4 *p) { return *p; }
+
+// Makes the compiler forget what it knows about a packed register array (no
+// instruction is emitted).  Used on loop-invariant packed parameters at the
+// top of each row iteration: without it the unpacked fp32 copies are hoisted
+// out of the loop and held live across it, which costs two registers per
+// packed dword and pushes the kernels into spilling.
+template <int N>
+__device__ __forceinline__ void keep_packed(u32x4 (&a)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) asm volatile("" : "+v"(a[k]));
+}
+
+// ---- wave64 reductions ---------------------------------------------------
+// DPP control words (GCN3/CDNA "data parallel primitives").
+constexpr int kDppQuadXor1 = 0xB1;      // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;      // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+constexpr int kDppRowBcast15 = 0x142;   // lane 15 of each row -> next row
+constexpr int kDppRowBcast31 = 0x143;   // lane 31 -> rows 2 and 3
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_take(float v) {
+    // Lanes outside ROW_MASK receive 0.
+    return as_f32((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Sum over each aligned group of 16 lanes; every lane gets its group's sum.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_take<kDppQuadXor1, 0xf>(v);
+    v += dpp_take<kDppQuadXor2, 0xf>(v);
+    v += dpp_take<kDppRowHalfMirror, 0xf>(v);
+    v += dpp_take<kDppRowMirror, 0xf>(v);
+    return v;
+}
+
+// Sum over each aligned group of LANES lanes (16, 32 or 64); every lane of the
+// group gets the sum.  The 64-lane form funnels the four DPP-row sums into
+// lane 63 with two row broadcasts and returns it through a scalar register,
+// so it costs no LDS traffic at all.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+    v = row16_sum(v);
+    if constexpr (LANES == 32) {
+        v += __shfl_xor(v, 16, kWaveSize);
+    } else if constexpr (LANES == 64) {
+        v += dpp_take<kDppRowBcast15, 0xa>(v);
+        v += dpp_take<kDppRowBcast31, 0xc>(v);
+        v = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 63));
+    }
+    return v;
+}
+
+// Adds, for every lane, the values held by the lanes that own the SAME columns
+// in the other rows of this wavefront (RPW rows per wavefront).
+template <int LANES>
+__device__ __forceinline__ float fold_rows_of_wave(float v) {
+    if constexpr (LANES <= 32) v += __shfl_xor(v, 32, kWaveSize);
+    if constexpr (LANES <= 16) v += __shfl_xor(v, 16, kWaveSize);
+    return v;
+}
+
+__device__ __forceinline__ int wave_id_in_block() {
+    return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+}
+
+// Adds this workgroup's per-lane column accumulators (acc[k][j] belongs to
+// column (k*LANES + l)*VEC + j) across the rows of each wavefront and across
+// wavefronts in fixed order, and writes one fp32 row of NSETS*C partial sums.
+template <typename G, int NSETS>
+__device__ __forceinline__ void flush_column_partials(float (&acc)[NSETS][G::CHUNKS][G::VEC],
+                                                      float *__restrict__ partial_row, float *lds) {
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS;
+    constexpr int C = VEC * LANES * CHUNKS;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s)
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[s][k][j] = fold_rows_of_wave<LANES>(acc[s][k][j]);
+
+    // wavefront 0 deposits, wavefronts 1.. add in turn: one fixed order
+    for (int wv = 0; wv < kRowWaves; ++wv) {
+        if (wave == wv && sub == 0) {
+#pragma unroll
+            for (int s = 0; s < NSETS; ++s)
+#pragma unroll
+                for (int k = 0; k < CHUNKS; ++k) {
+                    float *p = lds + s * C + (k * LANES + l) * VEC;
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) p[j] = (wv == 0) ? acc[s][k][j] : p[j] + acc[s][k][j];
+                }
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < NSETS * C; i += kRowThreads) partial_row[i] = lds[i];
+}
+
+}  // namespace ttn

@@ -1,0 +1,51 @@
+// Host-side plumbing shared by the C-ABI entry points: status + thread-local
+// error text, argument checks, cached device facts and the launch geometry
+// ("plan") that both the workspace queries and the launches derive from.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/teletron_norm.h"
+#include "norm_device.h"
+
+namespace ttn {
+
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Number of compute units of the current device (cached per device ordinal).
+int current_device_cus(int *status);
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline size_t elem_bytes(int dtype) { return dtype == TT_NORM_BF16 ? 2 : 4; }
+
+// Checks the last launch on this thread; returns TT_NORM_OK or TT_NORM_EHIP.
+int check_launch(const char *what);
+
+// ---- launch geometry -------------------------------------------------------
+// Every row kernel runs as a persistent 1-D grid of `batch * blocks_per_sample`
+// workgroups of kRowWaves wavefronts.  Workgroup i serves sample
+// i / blocks_per_sample only, and walks that sample's rows with stride
+// blocks_per_sample * kRowWaves * RPW, so per-sample parameters are loaded once
+// per workgroup and backward partial sums are naturally segmented by sample.
+
+struct RowPlan {
+    int rows_per_wave;       // RPW of the geometry
+    int blocks_per_sample;   // >= 1
+    int64_t blocks;          // batch * blocks_per_sample
+};
+
+// `blocks_per_cu`: how many workgroups per compute unit the kernel is tuned for.
+RowPlan make_row_plan(int64_t batch, int64_t rows_per_sample, int rows_per_wave,
+                      int blocks_per_cu, int cus);
+
+// Stage-2 reducer: partial[batch][blocks_per_sample][ncols] fp32 ->
+// out0[batch][C] (columns [0, C)) and, when ncols == 2C, out1[batch][C].
+int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch,
+                     int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
+                     hipStream_t stream);
+
+}  // namespace ttn

@@ -1,0 +1,203 @@
+// Status handling, device facts, launch geometry, the fixed-order column
+// reducer (stage 2 of every parameter-gradient reduction) and the streaming
+// copy used as the bandwidth yardstick.
+#include "norm_host.h"
+
+#include <atomic>
+#include <string.h>
+
+#include "norm_device.h"
+
+namespace ttn {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int current_device_cus(int *status) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cache[kMaxDevices];  // zero-initialised: 0 = unknown
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        *status = fail(TT_NORM_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+        return 0;
+    }
+    if (dev >= 0 && dev < kMaxDevices) {
+        int c = cache[dev].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    int cus = 0;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || cus <= 0) {
+        *status = fail(TT_NORM_EHIP, "hipDeviceGetAttribute(multiprocessor count): %s",
+                       hipGetErrorString(e));
+        return 0;
+    }
+    if (dev >= 0 && dev < kMaxDevices) cache[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TT_NORM_EHIP, "%s: %s", what, hipGetErrorString(e));
+    return TT_NORM_OK;
+}
+
+RowPlan make_row_plan(int64_t batch, int64_t rows_per_sample, int rows_per_wave,
+                      int blocks_per_cu, int cus) {
+    RowPlan p;
+    p.rows_per_wave = rows_per_wave;
+    const int64_t rows_per_block = (int64_t)kRowWaves * rows_per_wave;
+    const int64_t needed = (rows_per_sample + rows_per_block - 1) / rows_per_block;  // per sample
+    int64_t budget = ((int64_t)cus * blocks_per_cu) / batch;  // share of the persistent grid
+    if (budget < 1) budget = 1;
+    int64_t bps = needed < budget ? needed : budget;
+    if (bps < 1) bps = 1;
+    p.blocks_per_sample = (int)bps;
+    p.blocks = batch * bps;
+    return p;
+}
+
+// ---- stage 2: fixed-order column reduction ---------------------------------
+// partial[b][g][ncols] -> out[b][c].  A workgroup of 32 x 32 threads owns 32
+// adjacent columns of one sample; thread (tx, ty) adds partial rows ty, ty+32,
+// ... of column tx in ascending order, then one thread per column adds the 32
+// strands in ascending ty.  Every sum has one fixed association order, so the
+// result is bit-identical from run to run.
+constexpr int kRedCols = 32;
+constexpr int kRedStrands = 32;
+
+template <typename T>
+__device__ __forceinline__ void store_scalar(T *p, float v);
+template <>
+__device__ __forceinline__ void store_scalar<float>(float *p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_scalar<bf16_t>(bf16_t *p, float v) {
+    p->bits = (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
+    T *__restrict__ out0, T *__restrict__ out1, const float *__restrict__ partial,
+    int blocks_per_sample, int C, int ncols, int col_blocks) {
+    __shared__ float strands[kRedStrands][kRedCols + 1];
+    const int tx = threadIdx.x % kRedCols;
+    const int ty = threadIdx.x / kRedCols;
+    const int64_t b = blockIdx.x / col_blocks;
+    const int col = (int)(blockIdx.x % col_blocks) * kRedCols + tx;
+    float acc = 0.0f;
+    if (col < ncols) {
+        const float *p = partial + (b * blocks_per_sample) * (int64_t)ncols + col;
+        int g = ty;
+        // four loads in flight per thread; the additions stay in ascending-g order
+        for (; g + 3 * kRedStrands < blocks_per_sample; g += 4 * kRedStrands) {
+            const float v0 = p[(int64_t)g * ncols];
+            const float v1 = p[(int64_t)(g + kRedStrands) * ncols];
+            const float v2 = p[(int64_t)(g + 2 * kRedStrands) * ncols];
+            const float v3 = p[(int64_t)(g + 3 * kRedStrands) * ncols];
+            acc = (((acc + v0) + v1) + v2) + v3;
+        }
+        for (; g < blocks_per_sample; g += kRedStrands) acc += p[(int64_t)g * ncols];
+    }
+    strands[ty][tx] = acc;
+    __syncthreads();
+    if (ty == 0 && col < ncols) {
+        float s = strands[0][tx];
+#pragma unroll
+        for (int i = 1; i < kRedStrands; ++i) s += strands[i][tx];
+        if (col < C)
+            store_scalar<T>(out0 + b * C + col, s);
+        else
+            store_scalar<T>(out1 + b * C + (col - C), s);
+    }
+}
+
+int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch,
+                     int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
+                     hipStream_t stream) {
+    const int col_blocks = (int)((ncols + kRedCols - 1) / kRedCols);
+    const int64_t grid = batch * col_blocks;
+    if (grid > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "column reducer grid too large");
+    dim3 g((unsigned)grid), blk(kRedCols * kRedStrands);
+    if (dtype == TT_NORM_BF16)
+        colreduce_kernel<bf16_t><<<g, blk, 0, stream>>>((bf16_t *)out0, (bf16_t *)out1, partial,
+                                                        blocks_per_sample, (int)C, (int)ncols, col_blocks);
+    else
+        colreduce_kernel<float><<<g, blk, 0, stream>>>((float *)out0, (float *)out1, partial,
+                                                       blocks_per_sample, (int)C, (int)ncols, col_blocks);
+    return check_launch("column reducer launch");
+}
+
+// ---- streaming copy ----------------------------------------------------------
+__global__ __launch_bounds__(256) void stream_copy_kernel(u32x4 *__restrict__ dst,
+                                                          const u32x4 *__restrict__ src, size_t n16) {
+    // six 16-byte accesses in flight per lane, the same depth as one 3072-wide bf16 row
+    constexpr int kDepth = 6;
+    const size_t tile = (size_t)blockDim.x * kDepth;
+    for (size_t base = (size_t)blockIdx.x * tile; base < n16; base += (size_t)gridDim.x * tile) {
+        u32x4 v[kDepth];
+#pragma unroll
+        for (int k = 0; k < kDepth; ++k) {
+            const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
+            if (i < n16) v[k] = load16_stream(src + i);
+        }
+#pragma unroll
+        for (int k = 0; k < kDepth; ++k) {
+            const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
+            if (i < n16) store16_stream(dst + i, v[k]);
+        }
+    }
+}
+
+}  // namespace ttn
+
+using namespace ttn;
+
+extern "C" {
+
+int tt_norm_abi_version(void) { return TT_NORM_ABI_VERSION; }
+
+const char *tt_norm_status_string(int status) {
+    switch (status) {
+        case TT_NORM_OK: return "ok";
+        case TT_NORM_EINVAL: return "invalid argument";
+        case TT_NORM_EUNSUPPORTED: return "unsupported cols/dtype";
+        case TT_NORM_EALIGN: return "pointer not 16-byte aligned";
+        case TT_NORM_EWORKSPACE: return "workspace missing or too small";
+        case TT_NORM_EHIP: return "HIP runtime error";
+        default: return "unknown status";
+    }
+}
+
+const char *tt_norm_last_error(void) { return g_last_error; }
+
+int tt_norm_supported(int64_t cols, int dtype) {
+    if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F32) return 0;
+    return (cols == 128 || cols == 3072) ? 1 : 0;
+}
+
+int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
+    if (!dst || !src) return fail(TT_NORM_EINVAL, "stream_copy: null pointer");
+    if (bytes % 16) return fail(TT_NORM_EINVAL, "stream_copy: bytes (%zu) not a multiple of 16", bytes);
+    if (!aligned16(dst) || !aligned16(src)) return fail(TT_NORM_EALIGN, "stream_copy: unaligned pointer");
+    if (bytes == 0) return TT_NORM_OK;
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const size_t n16 = bytes / 16;
+    size_t blocks = (n16 + 256 * 6 - 1) / (256 * 6);
+    const size_t cap = (size_t)cus * 8;
+    if (blocks > cap) blocks = cap;
+    stream_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        (u32x4 *)dst, (const u32x4 *)src, n16);
+    return check_launch("stream copy launch");
+}
+
+}  // extern "C"

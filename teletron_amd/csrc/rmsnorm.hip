@@ -1,0 +1,286 @@
+// Fused RMSNorm for gfx950: forward, and a single-pass backward that produces
+// dx together with per-workgroup partial column sums for dweight.
+//
+// Math (rounding points follow the eager graph of
+// teletron/models/dit/dit_fusedlayers.py:360-370, "rnd" = round to the element
+// type, identity for fp32):
+//   forward   r = 1/sqrt(mean_c(x^2) + eps);  y = rnd(x*r);  out = rnd(y*w)
+//   backward  gy = rnd(g*w);  dx = rnd(gy*r - x * r^3 * mean_c(gy*x))
+//             dw[c] = sum_rows rnd(g * y)
+// HBM traffic per row: forward reads x, writes out (+4 B of rstd); backward
+// reads g and x, writes dx; dweight costs one fp32 row per workgroup.
+#include "norm_device.h"
+#include "norm_host.h"
+
+namespace ttn {
+
+template <typename T, int C>
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void rmsnorm_fwd_kernel(
+    T *__restrict__ out, float *__restrict__ rstd, const T *__restrict__ x,
+    const T *__restrict__ w, int64_t rows, float eps) {
+    using G = RowGeom<T, C>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;  // which of the wavefront's rows
+    const int l = lane % LANES;    // position inside the row
+    const int wave = wave_id_in_block();
+
+    u32x4 wr[CHUNKS];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) wr[k] = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
+
+    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(wr);
+        const int64_t row = grp * RPW + sub;
+        const bool ok = row < rows;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(x + row * C) + l;
+        u32x4 xr[CHUNKS];
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) ss = fmaf(v[j], v[j], ss);
+        }
+        ss = group_sum<LANES>(ss);
+        const float r = 1.0f / sqrtf(ss / (float)C + eps);
+        if (ok && l == 0) rstd[row] = r;
+
+        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC], wv[VEC];
+            E::unpack(xr[k], v);
+            E::unpack(wr[k], wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= r;
+            E::round(v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+            if (ok) store16_stream(po + k * LANES, E::pack(v));
+        }
+    }
+}
+
+// FROM_OUT = false: xin is the saved input x.
+// FROM_OUT = true : xin is the saved forward output; xhat is recovered as out/w.
+template <typename T, int C, bool FROM_OUT>
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void rmsnorm_bwd_kernel(
+    T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
+    const T *__restrict__ xin, const T *__restrict__ w, const float *__restrict__ rstd,
+    int64_t rows) {
+    using G = RowGeom<T, C>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    __shared__ float lds[C];
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+
+    u32x4 wr[CHUNKS];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) wr[k] = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
+
+    float acc[1][CHUNKS][VEC];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[0][k][j] = 0.0f;
+
+    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(wr);
+        const int64_t row = grp * RPW + sub;
+        const bool ok = row < rows;
+        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + row * C) + l;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + row * C) + l;
+        u32x4 gr[CHUNKS], xr[CHUNKS];
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            gr[k] = ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+            xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        }
+        const float r = ok ? rstd[row] : 0.0f;
+
+        // pass 1 over registers: row dot product  sum_c gy * xs
+        //   xs = x (native) or xhat = out / w (from the saved output)
+        float dot = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], xv[VEC], wv[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(xr[k], xv);
+            E::unpack(wr[k], wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] *= wv[j];
+            E::round(gv);  // gy materialised in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xs = FROM_OUT ? xv[j] * __builtin_amdgcn_rcpf(wv[j]) : xv[j];
+                dot = fmaf(gv[j], xs, dot);
+            }
+        }
+        dot = group_sum<LANES>(dot);
+        // Pass 2 re-derives gy from the packed registers instead of keeping 2*C/LANES
+        // fp32 values live across the reduction (registers buy occupancy here).
+        keep_packed(gr);
+        keep_packed(xr);
+        // dx = gy*r + xs*coef
+        const float coef = FROM_OUT ? -(r * (dot / (float)C)) : -((dot / (float)C) * r * r * r);
+
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], gy[VEC], xv[VEC], wv[VEC], o[VEC], y[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(xr[k], xv);
+            E::unpack(wr[k], wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gy[j] = gv[j] * wv[j];
+            E::round(gy);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float xs = FROM_OUT ? xv[j] * __builtin_amdgcn_rcpf(wv[j]) : xv[j];
+                o[j] = fmaf(xs, coef, gy[j] * r);
+                y[j] = FROM_OUT ? xs : xs * r;
+            }
+            if (ok) store16_stream(pd + k * LANES, E::pack(o));
+            E::round(y);  // y = normalised row in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
+            E::round(y);  // g*y materialised in the element type before the column sum
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[0][k][j] += y[j];
+        }
+    }
+    flush_column_partials<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds);
+}
+
+// ---- tuning: workgroups per compute unit of the persistent grids ------------
+template <typename T, int C>
+struct RmsTune {
+    static constexpr int kFwdBlocksPerCu = 8;
+    static constexpr int kBwdBlocksPerCu = 4;
+};
+
+template <typename T, int C>
+static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *w, int64_t rows,
+                             double eps, hipStream_t stream) {
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const RowPlan p = make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kFwdBlocksPerCu, cus);
+    rmsnorm_fwd_kernel<T, C><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+        (T *)out, rstd, (const T *)x, (const T *)w, rows, (float)eps);
+    return check_launch("rmsnorm forward launch");
+}
+
+template <typename T, int C>
+static RowPlan rmsnorm_backward_plan(int64_t rows, int cus) {
+    return make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kBwdBlocksPerCu, cus);
+}
+
+template <typename T, int C, bool FROM_OUT>
+static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin, const void *w,
+                              const float *rstd, int64_t rows, int dtype, void *ws, size_t ws_bytes,
+                              hipStream_t stream) {
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const RowPlan p = rmsnorm_backward_plan<T, C>(rows, cus);
+    const size_t need = (size_t)p.blocks * C * sizeof(float);
+    if (!ws || ws_bytes < need)
+        return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
+    rmsnorm_bwd_kernel<T, C, FROM_OUT><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, rows);
+    st = check_launch("rmsnorm backward launch");
+    if (st != TT_NORM_OK) return st;
+    return launch_colreduce(dw, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);
+}
+
+static int check_rms_args(const char *who, int64_t rows, int64_t cols, int dtype,
+                          std::initializer_list<const void *> ptrs) {
+    if (rows <= 0 || cols <= 0) return fail(TT_NORM_EINVAL, "%s: rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
+    if (!tt_norm_supported(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
+                    (long long)cols, dtype);
+    for (const void *p : ptrs) {
+        if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
+        if (!aligned16(p)) return fail(TT_NORM_EALIGN, "%s: pointer %p not 16-byte aligned", who, p);
+    }
+    return TT_NORM_OK;
+}
+
+}  // namespace ttn
+
+using namespace ttn;
+
+#define TTN_DISPATCH(dtype, cols, CALL)                          \
+    do {                                                         \
+        if ((dtype) == TT_NORM_BF16) {                           \
+            if ((cols) == 128) { CALL(bf16_t, 128); }            \
+            else { CALL(bf16_t, 3072); }                         \
+        } else {                                                 \
+            if ((cols) == 128) { CALL(float, 128); }             \
+            else { CALL(float, 3072); }                          \
+        }                                                        \
+    } while (0)
+
+extern "C" {
+
+int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight, int64_t rows,
+                       int64_t cols, double eps, int dtype, void *stream) {
+    int st = check_rms_args("tt_rmsnorm_forward", rows, cols, dtype, {out, x, weight});
+    if (st != TT_NORM_OK) return st;
+    if (!rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward: null rstd");
+#define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, rows, eps, (hipStream_t)stream)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+    if (rows <= 0 || !tt_norm_supported(cols, dtype)) return 0;
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return 0;
+#define CALL(T, C) return (size_t)rmsnorm_backward_plan<T, C>(rows, cus).blocks * C * sizeof(float)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x, const void *weight,
+                        const float *rstd, int64_t rows, int64_t cols, int dtype, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+    int st = check_rms_args("tt_rmsnorm_backward", rows, cols, dtype, {dx, dout, x, weight});
+    if (st != TT_NORM_OK) return st;
+    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
+#define CALL(T, C)                                                                                  \
+    return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, rows, dtype, workspace, \
+                                           workspace_bytes, (hipStream_t)stream)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, const void *out,
+                                 const void *weight, const float *rstd, int64_t rows, int64_t cols,
+                                 int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    int st = check_rms_args("tt_rmsnorm_backward_from_out", rows, cols, dtype, {dx, dout, out, weight});
+    if (st != TT_NORM_OK) return st;
+    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_from_out: null dweight/rstd");
+#define CALL(T, C)                                                                                   \
+    return rmsnorm_backward_t<T, C, true>(dx, dweight, dout, out, weight, rstd, rows, dtype, workspace, \
+                                          workspace_bytes, (hipStream_t)stream)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+}  // extern "C"

@@ -1,0 +1,330 @@
+"""GPU parity: the HIP kernels, called through the C ABI (teletron_amd.capi ->
+libteletron_norm.so), against the CPU oracle on identical seeded inputs.
+
+Bars (stated once, used everywhere below):
+  forward, bf16 : >= 99.9 % of elements bit-identical to eager and every element
+                  within 1 bf16 ulp, with one excusable exception: the kernels
+                  and eager sum a row in different orders, so the normalised
+                  value (y or xn) can flip by one ulp; eager then multiplies it
+                  (by w or 1+scale), re-rounds, and for AdaLN adds shift, which
+                  can turn that one ulp into 2-3 ulp of the result (or many, when
+                  the add cancels).  Such elements must lie within 2^-6 of the
+                  larger operand (|out| for RMSNorm, max(|xn*(1+scale)|, |shift|)
+                  for AdaLN) and number < 1e-4 of all elements;
+  forward, fp32 : rel 1e-5 (abs 1e-6);
+  gradients bf16: |got - want| <= 1e-3 + 1e-2 * |want| on every element
+                  (AdaLN dx: on all but 1e-5 of elements);
+  gradients fp32: rel 1e-4 / abs 1e-5 (column sums: rel 1e-4 of the column's L1 mass).
+"""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+from tests.golden_util import load_golden
+
+pytestmark = pytest.mark.gpu
+EPS = 1e-6
+
+
+@pytest.fixture(scope="module")
+def capi(gpu_device):
+    from teletron_amd import capi as c
+    c.lib()
+    return c
+
+
+def dev(d, device):
+    return {k: (v.to(device) if torch.is_tensor(v) else v) for k, v in d.items()}
+
+
+def assert_fwd_bf16(got, want, guard=None, what=""):
+    if guard is None:
+        guard = want.float().abs()
+    rep = O.compare_bf16_ulp(got.cpu(), want, cancel_scale=guard)
+    assert rep.n_gt1 == 0, (what, rep)
+    assert rep.n_excused <= 1e-4 * rep.n, (what, rep)
+    assert rep.frac_exact >= 0.999, (what, rep)
+
+
+def assert_grad_bf16(got, want, what="", allow=0.0):
+    frac = O.frac_outside(got.cpu(), want, 1e-2, 1e-3)
+    assert frac <= allow, (what, frac)
+
+
+def adaln_guard(d, eps=EPS):
+    """max(|p|, |shift|) per element from the oracle's staged forward."""
+    x, scale, shift = d["x"], d["scale"], d["shift"]
+    B, C = scale.shape
+    x3 = x.reshape(B, -1, C)
+    xn = torch.nn.functional.layer_norm(x3, (C,), None, None, eps)
+    p = xn * (1 + scale[:, None])
+    return torch.maximum(p.float().abs(), shift[:, None].float().abs().expand_as(p)).reshape(x.shape)
+
+
+# ------------------------------------------------------------------ goldens
+
+def test_golden_vectors(capi, gpu_device):
+    for name, d in load_golden().items():
+        g = dev(d, gpu_device)
+        if name.startswith("rms"):
+            out, rstd = capi.rmsnorm_forward(g["x"], g["weight"], EPS)
+            dx, dw = capi.rmsnorm_backward(g["grad"], g["x"], g["weight"], rstd)
+            got = {"out": out, "dx": dx, "dweight": dw}
+            guard = None
+        else:
+            out, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+            dx, ds, dh = capi.adaln_backward(g["grad"], g["x"], g["scale"], mean, rstd)
+            got = {"out": out, "dx": dx, "dscale": ds, "dshift": dh}
+            guard = adaln_guard(d) if d["is_bf16"] else None
+        for k, v in got.items():
+            if d["is_bf16"]:
+                if k == "out":
+                    assert_fwd_bf16(v, d[k], guard, f"{name}/{k}")
+                else:
+                    assert_grad_bf16(v, d[k], f"{name}/{k}", allow=1e-5 if k == "dx" else 0.0)
+            else:
+                torch.testing.assert_close(v.cpu(), d[k], rtol=1e-4, atol=1e-5, msg=f"{name}/{k}")
+
+
+# ------------------------------------------------------------------ RMSNorm
+
+@pytest.mark.parametrize("cols,rows", [(128, 1), (128, 3), (128, 4), (128, 4099), (128, 100003),
+                                       (3072, 1), (3072, 5), (3072, 1031), (3072, 9001)])
+def test_rmsnorm_bf16_vs_eager(capi, gpu_device, cols, rows):
+    d = O.make_rmsnorm_inputs((rows,), cols, torch.bfloat16, seed=100 + rows % 97)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    g = dev(d, gpu_device)
+    out, rstd = capi.rmsnorm_forward(g["x"], g["weight"], EPS)
+    assert_fwd_bf16(out, want_out, None, "out")
+    _, want_r = O.staged_rmsnorm_fwd(d["x"], d["weight"])
+    torch.testing.assert_close(rstd.cpu(), want_r.reshape(-1), rtol=1e-6, atol=0)
+    dx, dw = capi.rmsnorm_backward(g["grad"], g["x"], g["weight"], rstd)
+    assert_grad_bf16(dx, want_dx, "dx")
+    assert_grad_bf16(dw, want_dw, "dweight")
+    # dx is also nearly bit-identical to eager (same rounding points)
+    assert O.compare_bf16_ulp(dx.cpu(), want_dx).frac_exact > 0.99
+
+
+@pytest.mark.parametrize("cols,rows", [(128, 777), (3072, 8192 // 16)])
+def test_rmsnorm_fp32_vs_eager(capi, gpu_device, cols, rows):
+    d = O.make_rmsnorm_inputs((rows,), cols, torch.float32, seed=7)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    g = dev(d, gpu_device)
+    out, rstd = capi.rmsnorm_forward(g["x"], g["weight"], EPS)
+    torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-6)
+    dx, dw = capi.rmsnorm_backward(g["grad"], g["x"], g["weight"], rstd)
+    torch.testing.assert_close(dx.cpu(), want_dx, rtol=1e-4, atol=1e-5)
+    l1 = (d["grad"].abs() * want_out.abs()).sum(0)
+    assert ((dw.cpu() - want_dw).abs() <= 1e-4 * l1 + 1e-5).all()
+
+
+@pytest.mark.parametrize("cols,rows", [(128, 5001), (3072, 515)])
+def test_rmsnorm_backward_from_saved_output(capi, gpu_device, cols, rows):
+    """The reference-compatible entry point works from the forward OUTPUT."""
+    d = O.make_rmsnorm_inputs((rows,), cols, torch.bfloat16, seed=5)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    g = dev(d, gpu_device)
+    out, rstd = capi.rmsnorm_forward(g["x"], g["weight"], EPS)
+    dx, dw = capi.rmsnorm_backward(g["grad"], out, g["weight"], rstd, from_out=True)
+    # xhat is recovered from a bf16 tensor: one extra bf16 rounding on xhat, so the
+    # bar is the gradient bar on >= 99.9 % of elements, 3x the bar on the rest
+    assert O.frac_outside(dx.cpu(), want_dx, 1e-2, 1e-3) < 1e-3
+    assert O.frac_outside(dx.cpu(), want_dx, 3e-2, 3e-3) == 0.0
+    assert O.frac_outside(dw.cpu(), want_dw, 3e-2, 3e-3) == 0.0
+
+
+# -------------------------------------------------------------------- AdaLN
+
+@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 7), (1, 2053), (4, 333), (3, 1), (5, 1001), (300, 2)])
+def test_adaln_bf16_vs_eager(capi, gpu_device, batch, seq):
+    d = O.make_adaln_inputs(batch, seq, 3072, torch.bfloat16, seed=200 + seq % 89, sigma=1.5)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    g = dev(d, gpu_device)
+    out, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    assert_fwd_bf16(out, want_out, adaln_guard(d), "out")
+    _, want_mu, want_r = O.staged_adaln_fwd(d["x"], d["scale"], d["shift"])
+    torch.testing.assert_close(rstd.cpu(), want_r.reshape(-1), rtol=2e-6, atol=0)
+    torch.testing.assert_close(mean.cpu(), want_mu.reshape(-1), rtol=0, atol=2e-6)
+    dx, ds, dh = capi.adaln_backward(g["grad"], g["x"], g["scale"], mean, rstd)
+    assert_grad_bf16(dx, want_dx, "dx", allow=1e-5)
+    assert_grad_bf16(ds, want_ds, "dscale")
+    assert_grad_bf16(dh, want_dh, "dshift")
+
+
+def test_adaln_fp32_vs_eager(capi, gpu_device):
+    d = O.make_adaln_inputs(3, 171, 3072, torch.float32, seed=9)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    g = dev(d, gpu_device)
+    out, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-5)
+    dx, ds, dh = capi.adaln_backward(g["grad"], g["x"], g["scale"], mean, rstd)
+    torch.testing.assert_close(dx.cpu(), want_dx, rtol=1e-4, atol=1e-5)
+    l1 = d["grad"].abs().sum(1)
+    assert ((dh.cpu() - want_dh).abs() <= 1e-4 * l1 + 1e-5).all()
+    assert ((ds.cpu() - want_ds).abs() <= 1e-4 * 3 * l1 + 1e-5).all()
+
+
+def test_adaln_reference_compatible_entry_points(capi, gpu_device):
+    """forward that also writes x_norm + backward from x_norm (what the
+    reference's autograd class saves)."""
+    d = O.make_adaln_inputs(2, 409, 3072, torch.bfloat16, seed=31)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    g = dev(d, gpu_device)
+    out, xn, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS, want_xnorm=True)
+    out2, mean, rstd2 = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    assert torch.equal(out, out2) and torch.equal(rstd, rstd2)
+    want_xn = torch.nn.functional.layer_norm(d["x"], (3072,), None, None, EPS)
+    rep = O.compare_bf16_ulp(xn.cpu(), want_xn)
+    assert rep.n_gt1 == 0 and rep.frac_exact > 0.999
+    dx, ds, dh = capi.adaln_backward(g["grad"], xn, g["scale"], None, rstd, from_xnorm=True)
+    assert O.frac_outside(dx.cpu(), want_dx, 1e-2, 1e-3) < 1e-3     # xhat known to bf16 only
+    assert O.frac_outside(dx.cpu(), want_dx, 3e-2, 3e-3) == 0.0
+    assert_grad_bf16(ds, want_ds, "dscale")
+    assert_grad_bf16(dh, want_dh, "dshift")
+
+
+# -------------------------------------------- properties at the full shapes
+
+def _full_rows():
+    return 118800
+
+
+def test_full_size_rmsnorm_properties(capi, gpu_device):
+    """118 800 x 3072 bf16: determinism, exact linearity in the upstream grad,
+    and agreement with eager on a strided sample of rows."""
+    rows, C = _full_rows(), 3072
+    gen = torch.Generator(device=gpu_device).manual_seed(0)
+    x = torch.randn(rows, C, device=gpu_device, generator=gen).bfloat16()
+    grad = torch.randn(rows, C, device=gpu_device, generator=gen).bfloat16()
+    w = (1 + 0.02 * torch.randn(C, device=gpu_device, generator=gen)).bfloat16()
+    out, rstd = capi.rmsnorm_forward(x, w, EPS)
+    out2, rstd2 = capi.rmsnorm_forward(x, w, EPS)
+    assert torch.equal(out, out2) and torch.equal(rstd, rstd2)
+    dx, dw = capi.rmsnorm_backward(grad, x, w, rstd)
+    dx2, dw2 = capi.rmsnorm_backward(grad, x, w, rstd)
+    assert torch.equal(dx, dx2) and torch.equal(dw, dw2)           # deterministic reduction
+    dx4, dw4 = capi.rmsnorm_backward(grad * 4, x, w, rstd)          # exact power-of-two scaling
+    assert torch.equal(dx4, dx * 4)
+    torch.testing.assert_close(dw4.float(), dw.float() * 4, rtol=2 ** -7, atol=0)
+    # sampled rows against eager on the CPU
+    idx = torch.arange(0, rows, 997, device=gpu_device)
+    xs, gs = x[idx].cpu(), grad[idx].cpu()
+    want_out, want_dx, _ = O.eager_rmsnorm_fwd_bwd(xs, w.cpu(), gs)
+    assert_fwd_bf16(out[idx], want_out, None, "out rows")
+    assert_grad_bf16(dx[idx], want_dx, "dx rows")
+    # dweight against an independent fp32 column reduction on the GPU (torch ops)
+    y = (x.float() * rstd[:, None]).bfloat16()
+    want_dw = (grad * y).float().sum(0)
+    assert O.frac_outside(dw.cpu(), want_dw.cpu(), 1e-2, 1e-3) == 0.0
+
+
+def test_full_size_adaln_properties(capi, gpu_device):
+    rows, C = _full_rows(), 3072
+    gen = torch.Generator(device=gpu_device).manual_seed(1)
+    x = torch.randn(1, rows, C, device=gpu_device, generator=gen).bfloat16()
+    grad = torch.randn(1, rows, C, device=gpu_device, generator=gen).bfloat16()
+    scale = (0.1 * torch.randn(1, C, device=gpu_device, generator=gen)).bfloat16()
+    shift = (0.1 * torch.randn(1, C, device=gpu_device, generator=gen)).bfloat16()
+    out, mean, rstd = capi.adaln_forward(x, scale, shift, EPS)
+    out2, _, _ = capi.adaln_forward(x, scale, shift, EPS)
+    assert torch.equal(out, out2)
+    dx, ds, dh = capi.adaln_backward(grad, x, scale, mean, rstd)
+    dx2, ds2, dh2 = capi.adaln_backward(grad, x, scale, mean, rstd)
+    assert torch.equal(dx, dx2) and torch.equal(ds, ds2) and torch.equal(dh, dh2)
+    dx4, ds4, dh4 = capi.adaln_backward(grad * 4, x, scale, mean, rstd)
+    assert torch.equal(dx4, dx * 4)
+    # LayerNorm backward is orthogonal to the ones vector: row sums of dx vanish
+    # up to bf16 rounding of 3072 outputs (|dx| ~ 1 => noise ~ 2^-9 * sqrt(3072) ~ 0.1)
+    assert dx.float().sum(-1).abs().max() < 0.5
+    # dshift = column sums of the upstream gradient
+    want_dh = grad.float().sum(1)
+    assert O.frac_outside(dh.cpu(), want_dh.cpu(), 1e-2, 1e-3) == 0.0
+    idx = torch.arange(0, rows, 991, device=gpu_device)
+    d = {"x": x[:, idx].cpu(), "scale": scale.cpu(), "shift": shift.cpu(), "grad": grad[:, idx].cpu()}
+    want_out, want_dx, _, _ = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    assert_fwd_bf16(out[:, idx], want_out, adaln_guard(d), "out rows")
+    assert_grad_bf16(dx[:, idx], want_dx, "dx rows", allow=1e-5)
+
+
+def test_qk_norm_shape_one_cp_rank(capi, gpu_device):
+    """q of one CP=4 rank: [1, 29700, 24, 128] bf16 = 712 800 rows of 128."""
+    d = O.make_rmsnorm_inputs((1, 29700, 24), 128, torch.bfloat16, seed=0)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    g = dev(d, gpu_device)
+    out, rstd = capi.rmsnorm_forward(g["x"], g["weight"], EPS)
+    assert_fwd_bf16(out, want_out, None, "out")
+    dx, dw = capi.rmsnorm_backward(g["grad"], g["x"], g["weight"], rstd)
+    assert_grad_bf16(dx, want_dx, "dx")
+    assert_grad_bf16(dw, want_dw, "dweight")
+
+
+def test_batched_per_sample_modulation_chain(capi, gpu_device):
+    """batch 4 x (10800 + 256) tokens, sigma 2, distinct modulation per sample:
+    AdaLN then RMSNorm(3072), forward and backward of the chain."""
+    B, S, C = 4, 11056, 3072
+    d = O.make_adaln_inputs(B, S, C, torch.bfloat16, seed=0, sigma=2.0)
+    w = (1 + 0.02 * torch.randn(C, generator=torch.Generator().manual_seed(3))).bfloat16()
+    xr = d["x"].clone().requires_grad_(True)
+    sc = d["scale"].clone().requires_grad_(True)
+    sh = d["shift"].clone().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    y = O.eager_adaln(xr, sc, sh, EPS)
+    z = O.eager_rmsnorm(y, wr, EPS)
+    z.backward(d["grad"])
+    g = dev(d, gpu_device)
+    wg = w.to(gpu_device)
+    y_g, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    z_g, rstd2 = capi.rmsnorm_forward(y_g, wg, EPS)
+    assert_fwd_bf16(y_g, y.detach(), adaln_guard(d), "adaln out")
+    # z sees y's occasional 1-ulp differences re-normalised: same bar, exact fraction relaxed
+    rep = O.compare_bf16_ulp(z_g.cpu(), z.detach())
+    assert rep.frac_exact > 0.995 and O.frac_outside(z_g.cpu(), z.detach(), 1e-2, 1e-3) < 1e-5
+    dy, dw = capi.rmsnorm_backward(g["grad"], y_g, wg, rstd2)
+    dx, ds, dh = capi.adaln_backward(dy, g["x"], g["scale"], mean, rstd)
+    assert_grad_bf16(dw, wr.grad, "dweight")
+    assert_grad_bf16(dx, xr.grad, "dx", allow=1e-4)
+    assert_grad_bf16(ds, sc.grad, "dscale")
+    assert_grad_bf16(dh, sh.grad, "dshift")
+
+
+# ---------------------------------------------------------------- boundary
+
+def test_non_default_stream_and_output_reuse(capi, gpu_device):
+    d = dev(O.make_rmsnorm_inputs((4096,), 3072, torch.bfloat16, seed=1), gpu_device)
+    ref, _ = capi.rmsnorm_forward(d["x"], d["weight"], EPS)
+    side = torch.cuda.Stream(device=gpu_device)
+    side.wait_stream(torch.cuda.current_stream(gpu_device))
+    with torch.cuda.stream(side):
+        out, _ = capi.rmsnorm_forward(d["x"], d["weight"], EPS)
+    side.synchronize()
+    assert torch.equal(out, ref)
+
+
+def test_error_statuses(capi, gpu_device):
+    L = capi.lib()
+    x = torch.zeros(8, 3072, dtype=torch.bfloat16, device=gpu_device)
+    w = torch.ones(3072, dtype=torch.bfloat16, device=gpu_device)
+    r = torch.zeros(8, dtype=torch.float32, device=gpu_device)
+    vp = lambda t, off=0: ctypes.c_void_p(t.data_ptr() + off)
+    # unsupported column count
+    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), 8, 100, 1e-6, 0, None) == 2
+    assert b"cols=100" in L.tt_norm_last_error()
+    # unsupported dtype
+    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), 8, 3072, 1e-6, 7, None) == 2
+    # misaligned pointer
+    assert L.tt_rmsnorm_forward(vp(x, 2), vp(r), vp(x), vp(w), 4, 3072, 1e-6, 0, None) == 3
+    # null pointer / bad sizes
+    assert L.tt_rmsnorm_forward(None, vp(r), vp(x), vp(w), 8, 3072, 1e-6, 0, None) == 1
+    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), 0, 3072, 1e-6, 0, None) == 1
+    # workspace too small
+    need = L.tt_rmsnorm_backward_workspace_bytes(8, 3072, 0)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+    assert L.tt_rmsnorm_backward(vp(x), vp(w), vp(x), vp(x), vp(w), vp(r), 8, 3072, 0, vp(ws), need - 1, None) == 4
+    assert L.tt_rmsnorm_backward(vp(x), vp(w), vp(x), vp(x), vp(w), vp(r), 8, 3072, 0, None, 0, None) == 4
+    with pytest.raises(capi.NormError):
+        capi.rmsnorm_forward(torch.zeros(4, 256, dtype=torch.bfloat16, device=gpu_device),
+                             torch.ones(256, dtype=torch.bfloat16, device=gpu_device), EPS)
+    torch.cuda.synchronize()
