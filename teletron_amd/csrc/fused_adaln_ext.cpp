@@ -1,0 +1,144 @@
+// Python module `fused_adaln`: the two functions of the reference's module of
+// the same name, with the same argument order
+// (teletron_op/fused_adaln/adaln_ops.cpp:6-15,29-38,52-60), plus the native
+// pair that saves row statistics instead of a second full-size tensor.
+// scale/shift may hold one row per sample ([batch, cols]); rows are then
+// grouped by sample, rows/batch consecutive rows each.
+#include "torch_glue.h"
+
+using namespace ttn_glue;
+
+struct AdalnShape {
+    int64_t batch, rows_per_sample;
+    int dt;
+};
+
+static AdalnShape adaln_shape(const torch::Tensor &x, const torch::Tensor &scale, int64_t rows, int64_t cols) {
+    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    TORCH_CHECK(scale.numel() > 0 && scale.numel() % cols == 0, "scale has ", scale.numel(),
+                " elements, not a multiple of cols=", cols);
+    const int64_t batch = scale.numel() / cols;
+    TORCH_CHECK(rows % batch == 0, "rows=", rows, " is not a multiple of the ", batch, " modulation rows");
+    return {batch, rows / batch, dtype_code(x, "input")};
+}
+
+void torch_launch_adaln_forward(torch::Tensor &output, torch::Tensor &x_norm, const torch::Tensor &input,
+                                const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                int64_t cols, double epsilon, torch::Tensor &inv_variance) {
+    const auto dev = input.device();
+    for (auto *t : {&output, &x_norm, &inv_variance}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&input, &scale, &shift}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(input, scale, rows, cols);
+    const auto st = input.scalar_type();
+    check_elems(input, rows * cols, st, "input");
+    check_elems(output, rows * cols, st, "output");
+    check_elems(x_norm, rows * cols, st, "x_norm");
+    check_elems(shift, scale.numel(), st, "shift");
+    check_elems(scale, scale.numel(), st, "scale");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_adaln_forward_xnorm(output.data_ptr(), x_norm.data_ptr(), inv_variance.data_ptr<float>(),
+                                    input.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch,
+                                    s.rows_per_sample, cols, epsilon, s.dt, current_stream(input)),
+             "tt_adaln_forward_xnorm");
+}
+
+void torch_launch_adaln_forward_stats(torch::Tensor &output, const torch::Tensor &input,
+                                      const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                      int64_t cols, double epsilon, torch::Tensor &mean,
+                                      torch::Tensor &inv_variance) {
+    const auto dev = input.device();
+    for (auto *t : {&output, &mean, &inv_variance}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&input, &scale, &shift}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(input, scale, rows, cols);
+    const auto st = input.scalar_type();
+    check_elems(input, rows * cols, st, "input");
+    check_elems(output, rows * cols, st, "output");
+    check_elems(shift, scale.numel(), st, "shift");
+    check_elems(scale, scale.numel(), st, "scale");
+    check_elems(mean, rows, at::kFloat, "mean");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_adaln_forward(output.data_ptr(), mean.data_ptr<float>(), inv_variance.data_ptr<float>(),
+                              input.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch, s.rows_per_sample,
+                              cols, epsilon, s.dt, current_stream(input)),
+             "tt_adaln_forward");
+}
+
+static void adaln_backward_impl(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
+                                const torch::Tensor &dout, const torch::Tensor &saved,
+                                const torch::Tensor &scale, const torch::Tensor *mean,
+                                const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    const auto dev = dout.device();
+    for (auto *t : {&dinp, &dscale, &dshift}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&dout, &saved, &scale, &inv_variance}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(dout, scale, rows, cols);
+    const auto st = dout.scalar_type();
+    check_elems(dout, rows * cols, st, "dout");
+    check_elems(dinp, rows * cols, st, "dinp");
+    check_elems(saved, rows * cols, st, mean ? "input" : "x_norm");
+    check_elems(scale, scale.numel(), st, "scale");
+    check_elems(dscale, scale.numel(), st, "dscale");
+    check_elems(dshift, scale.numel(), st, "dshift");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    if (mean) {
+        check_dense_on(*mean, dev, "mean");
+        check_elems(*mean, rows, at::kFloat, "mean");
+    }
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_adaln_backward_workspace_bytes(s.batch, s.rows_per_sample, cols, s.dt);
+    TORCH_CHECK(need > 0, "unsupported AdaLN shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    if (mean)
+        raise_on(tt_adaln_backward(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(),
+                                   saved.data_ptr(), scale.data_ptr(), mean->data_ptr<float>(),
+                                   inv_variance.data_ptr<float>(), s.batch, s.rows_per_sample, cols, s.dt,
+                                   ws.data_ptr(), need, current_stream(dout)),
+                 "tt_adaln_backward");
+    else
+        raise_on(tt_adaln_backward_from_xnorm(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(),
+                                              dout.data_ptr(), saved.data_ptr(), scale.data_ptr(),
+                                              inv_variance.data_ptr<float>(), s.batch, s.rows_per_sample, cols,
+                                              s.dt, ws.data_ptr(), need, current_stream(dout)),
+                 "tt_adaln_backward_from_xnorm");
+}
+
+// Reference contract: x_norm is what torch_launch_adaln_forward wrote to `x_norm`.
+void torch_launch_adaln_backward(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
+                                 const torch::Tensor &dout, const torch::Tensor &x_norm,
+                                 const torch::Tensor &scale, const torch::Tensor &inv_variance, int64_t rows,
+                                 int64_t cols) {
+    adaln_backward_impl(dinp, dscale, dshift, dout, x_norm, scale, nullptr, inv_variance, rows, cols);
+}
+
+// Native contract: `input`, `mean`, `inv_variance` as seen / written by torch_launch_adaln_forward_stats.
+void torch_launch_adaln_backward_x(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
+                                   const torch::Tensor &dout, const torch::Tensor &input,
+                                   const torch::Tensor &scale, const torch::Tensor &mean,
+                                   const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    adaln_backward_impl(dinp, dscale, dshift, dout, input, scale, &mean, inv_variance, rows, cols);
+}
+
+PYBIND11_MODULE(fused_adaln, m) {
+    m.def("torch_launch_adaln_forward", &torch_launch_adaln_forward, "AdaLN forward kernel");
+    m.def("torch_launch_adaln_backward", &torch_launch_adaln_backward,
+          "AdaLN backward kernel (from the saved normalised rows)");
+    m.def("torch_launch_adaln_forward_stats", &torch_launch_adaln_forward_stats,
+          "AdaLN forward kernel that saves mean and inv_variance instead of x_norm");
+    m.def("torch_launch_adaln_backward_x", &torch_launch_adaln_backward_x,
+          "AdaLN backward kernel (from the saved input and statistics)");
+    m.def("supported", [](int64_t cols, const torch::Tensor &like) {
+        return tt_norm_supported(cols, like.scalar_type() == at::kBFloat16 ? TT_NORM_BF16
+                                       : like.scalar_type() == at::kFloat  ? TT_NORM_F32 : -1) != 0;
+    }, "whether the kernels are built for this column count and dtype");
+}
+
+// Same operator namespace as the reference registers (adaln_ops.cpp:62-65).
+TORCH_LIBRARY(layernorm_block_smem, m) {
+    m.def("torch_launch_adaln_forward(Tensor(a!) output, Tensor(b!) x_norm, Tensor input, Tensor scale, "
+          "Tensor shift, int rows, int cols, float epsilon, Tensor(c!) inv_variance) -> ()",
+          &torch_launch_adaln_forward);
+    m.def("torch_launch_adaln_backward(Tensor(a!) dinp, Tensor(b!) dscale, Tensor(c!) dshift, Tensor dout, "
+          "Tensor x_norm, Tensor scale, Tensor inv_variance, int rows, int cols) -> ()",
+          &torch_launch_adaln_backward);
+}

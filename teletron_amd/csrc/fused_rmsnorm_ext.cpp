@@ -1,0 +1,95 @@
+// Python module `fused_rmsnorm`: the two functions of the reference's module of
+// the same name, with the same argument order
+// (teletron_op/fused_rmsnorm/rms_ops.cpp:6-13,25-33,47-55), plus the native
+// backward that works from the saved input.  Unlike the reference glue, every
+// argument is checked, the launch goes to PyTorch's current stream, and a
+// failed launch raises.
+#include "torch_glue.h"
+
+using namespace ttn_glue;
+
+// output[rows, cols] = rmsnorm(input) * weight;  inv_variance[rows] = 1/rms  (fp32)
+void torch_launch_rms_forward(torch::Tensor &output, const torch::Tensor &input,
+                              const torch::Tensor &weight, int64_t rows, int64_t cols, double epsilon,
+                              torch::Tensor &inv_variance) {
+    const auto dev = input.device();
+    check_dense_on(input, dev, "input");
+    check_dense_on(output, dev, "output");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(input, "input");
+    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    check_elems(input, rows * cols, input.scalar_type(), "input");
+    check_elems(output, rows * cols, input.scalar_type(), "output");
+    check_elems(weight, cols, input.scalar_type(), "weight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_rmsnorm_forward(output.data_ptr(), inv_variance.data_ptr<float>(), input.data_ptr(),
+                                weight.data_ptr(), rows, cols, epsilon, dt, current_stream(input)),
+             "tt_rmsnorm_forward");
+}
+
+static void rms_backward_impl(torch::Tensor &dinp, torch::Tensor &dweight, const torch::Tensor &dout,
+                              const torch::Tensor &saved, const torch::Tensor &weight,
+                              const torch::Tensor &inv_variance, int64_t rows, int64_t cols,
+                              bool saved_is_output) {
+    const auto dev = dout.device();
+    check_dense_on(dout, dev, "dout");
+    check_dense_on(dinp, dev, "dinp");
+    check_dense_on(dweight, dev, "dweight");
+    check_dense_on(saved, dev, saved_is_output ? "x_norm" : "input");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(dout, "dout");
+    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    check_elems(dout, rows * cols, dout.scalar_type(), "dout");
+    check_elems(dinp, rows * cols, dout.scalar_type(), "dinp");
+    check_elems(saved, rows * cols, dout.scalar_type(), saved_is_output ? "x_norm" : "input");
+    check_elems(weight, cols, dout.scalar_type(), "weight");
+    check_elems(dweight, cols, dout.scalar_type(), "dweight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_rmsnorm_backward_workspace_bytes(rows, cols, dt);
+    TORCH_CHECK(need > 0, "unsupported RMSNorm shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    auto fn = saved_is_output ? tt_rmsnorm_backward_from_out : tt_rmsnorm_backward;
+    raise_on(fn(dinp.data_ptr(), dweight.data_ptr(), dout.data_ptr(), saved.data_ptr(), weight.data_ptr(),
+                inv_variance.data_ptr<float>(), rows, cols, dt, ws.data_ptr(), need, current_stream(dout)),
+             saved_is_output ? "tt_rmsnorm_backward_from_out" : "tt_rmsnorm_backward");
+}
+
+// Reference contract: x_norm is the tensor torch_launch_rms_forward wrote to `output`.
+void torch_launch_rms_backward(torch::Tensor &dinp, torch::Tensor &dweight, const torch::Tensor &dout,
+                               const torch::Tensor &x_norm, const torch::Tensor &weight,
+                               const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    rms_backward_impl(dinp, dweight, dout, x_norm, weight, inv_variance, rows, cols, true);
+}
+
+// Native contract: `input` is the tensor that was normalised (forward then keeps no copy of its output).
+void torch_launch_rms_backward_x(torch::Tensor &dinp, torch::Tensor &dweight, const torch::Tensor &dout,
+                                 const torch::Tensor &input, const torch::Tensor &weight,
+                                 const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    rms_backward_impl(dinp, dweight, dout, input, weight, inv_variance, rows, cols, false);
+}
+
+PYBIND11_MODULE(fused_rmsnorm, m) {
+    m.def("torch_launch_rms_forward", &torch_launch_rms_forward, "RMSNorm forward kernel");
+    m.def("torch_launch_rms_backward", &torch_launch_rms_backward,
+          "RMSNorm backward kernel (from the saved forward output)");
+    m.def("torch_launch_rms_backward_x", &torch_launch_rms_backward_x,
+          "RMSNorm backward kernel (from the saved input)");
+    m.def("supported", [](int64_t cols, const torch::Tensor &like) {
+        return tt_norm_supported(cols, like.scalar_type() == at::kBFloat16 ? TT_NORM_BF16
+                                       : like.scalar_type() == at::kFloat  ? TT_NORM_F32 : -1) != 0;
+    }, "whether the kernels are built for this column count and dtype");
+}
+
+// Same operator namespace as the reference registers (rms_ops.cpp:58-61).
+TORCH_LIBRARY(Fused_RMSNorm, m) {
+    m.def("torch_launch_rms_forward(Tensor(a!) output, Tensor input, Tensor weight, int rows, int cols, "
+          "float epsilon, Tensor(b!) inv_variance) -> ()",
+          &torch_launch_rms_forward);
+    m.def("torch_launch_rms_backward(Tensor(a!) dinp, Tensor(b!) dweight, Tensor dout, Tensor x_norm, "
+          "Tensor weight, Tensor inv_variance, int rows, int cols) -> ()",
+          &torch_launch_rms_backward);
+}

@@ -1,0 +1,327 @@
+"""Host-side operator interface of the fused normalization path.
+
+Exposes the names HunyuanVideo blocks import from the reference's
+teletron/models/dit/dit_fusedlayers.py -- AdaLNModelFunction (:59),
+AdaLNCustom (:139), FusedAdaLayerNormZero (:155), FusedAdaLayerNormZeroSingle
+(:226), RMSNormModelFunction (:274), Get_RMSNorm (:350), FP32LayerNorm (:48) --
+with the same call signatures, argument meaning, returned gradients and
+ValueErrors, backed by the gfx950 kernels.
+
+What differs from the reference, on purpose:
+  * the autograd functions keep the INPUT and per-row statistics for backward
+    (the reference keeps a second full-size tensor), so forward writes one
+    tensor and backward is a single pass plus a fixed-order reducer;
+  * scale/shift may carry one row per sample ([B, C]) and their gradients come
+    back per sample, which is what the eager formula at :223 computes; the
+    reference kernels only handle a single modulation row;
+  * both operators accept 128 and 3072 columns, bf16 and fp32;
+  * nothing here falls back silently: with FUSED_KERNELS on, a missing
+    extension or a non-GPU tensor raises.  The eager branches below exist only
+    because the reference modules select eager math when FUSED_KERNELS is off.
+"""
+from __future__ import annotations
+
+import logging
+import os
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.autograd import Function
+
+log = logging.getLogger(__name__)
+log.addHandler(logging.NullHandler())
+
+try:  # same guard as dit_fusedlayers.py:35-45, but the reason is kept for the error message
+    from teletron_amd.ext import fused_adaln, fused_rmsnorm
+    _IMPORT_ERROR: Optional[BaseException] = None
+except ImportError as exc:  # pragma: no cover - exercised only on an unbuilt tree
+    fused_adaln = None
+    fused_rmsnorm = None
+    _IMPORT_ERROR = exc
+    log.warning("fused_adaln / fused_rmsnorm extensions not importable (%s); "
+                "build them with `python -m teletron_amd.build`.", exc)
+
+SUPPORTED_COLS = (128, 3072)
+
+
+def fused_kernels_available() -> bool:
+    return fused_adaln is not None and fused_rmsnorm is not None
+
+
+def fused_kernels_requested() -> bool:
+    """The reference's switch: env FUSED_KERNELS parsed as an int (dit_fusedlayers.py:364-365)."""
+    flag = os.environ.get("FUSED_KERNELS")
+    return bool(int(flag)) if flag else False
+
+
+def _require_extension(mod, name: str):
+    if mod is None:
+        raise RuntimeError(f"{name} extension is not built/importable ({_IMPORT_ERROR}); "
+                           "run `python -m teletron_amd.build`")
+    return mod
+
+
+def _require_gpu(t: torch.Tensor, what: str):
+    if not t.is_cuda:
+        raise ValueError(f"{what}: fused kernels need a GPU tensor, got device {t.device}")
+
+
+class FP32LayerNorm(nn.LayerNorm):
+    """LayerNorm evaluated in fp32 and cast back (dit_fusedlayers.py:48-57)."""
+
+    def forward(self, inputs: torch.Tensor) -> torch.Tensor:
+        w = None if self.weight is None else self.weight.float()
+        b = None if self.bias is None else self.bias.float()
+        return F.layer_norm(inputs.float(), self.normalized_shape, w, b, self.eps).to(inputs.dtype)
+
+
+class AdaLNModelFunction(Function):
+    """out = LayerNorm(x) * (1 + scale) + shift, no LayerNorm affine.
+
+    apply(x, scale, shift, epsilon, cols) -> out, with gradients for x, scale
+    and shift (dit_fusedlayers.py:66,108).  x is [..., cols]; scale and shift are
+    [cols] or [B, cols] with B == x.shape[0] (one modulation row per sample).
+    """
+
+    @staticmethod
+    def forward(ctx, x, scale, shift, epsilon, cols):
+        ext = _require_extension(fused_adaln, "fused_adaln")
+        _require_gpu(x, "AdaLNModelFunction")
+        x = x.contiguous()
+        scale_c = scale.contiguous()
+        shift_c = shift.contiguous()
+        if cols not in SUPPORTED_COLS or x.numel() == 0 or x.numel() % cols != 0:
+            raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols} "
+                             f"or unsupported cols (supported: {SUPPORTED_COLS})")
+        rows = x.numel() // cols
+        if scale_c.numel() % cols != 0 or shift_c.numel() != scale_c.numel():
+            raise ValueError(f"scale/shift sizes {scale_c.numel()}/{shift_c.numel()} do not match cols {cols}")
+        batch = scale_c.numel() // cols
+        if batch > 1 and (x.dim() < 2 or x.shape[0] != batch):
+            raise ValueError(f"{batch} modulation rows need x.shape[0] == {batch}, got {tuple(x.shape)}")
+        if scale_c.dtype != x.dtype or shift_c.dtype != x.dtype:
+            scale_c, shift_c = scale_c.to(x.dtype), shift_c.to(x.dtype)
+
+        out = torch.empty_like(x)
+        mean = torch.empty(rows, device=x.device, dtype=torch.float32)
+        invvar = torch.empty(rows, device=x.device, dtype=torch.float32)
+        ext.torch_launch_adaln_forward_stats(out, x, scale_c, shift_c, rows, cols, float(epsilon), mean, invvar)
+        ctx.save_for_backward(x, scale_c, mean, invvar)
+        ctx.rows, ctx.cols = rows, cols
+        ctx.mod_shape, ctx.mod_dtype = scale.shape, scale.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, scale_c, mean, invvar = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if grad_output.dtype != x.dtype:
+            grad_output = grad_output.to(x.dtype)
+        grad_input = torch.empty_like(x)
+        grad_scale = torch.empty_like(scale_c)
+        grad_shift = torch.empty_like(scale_c)
+        fused_adaln.torch_launch_adaln_backward_x(grad_input, grad_scale, grad_shift, grad_output, x, scale_c,
+                                                  mean, invvar, ctx.rows, ctx.cols)
+        grad_scale = grad_scale.reshape(ctx.mod_shape).to(ctx.mod_dtype)
+        grad_shift = grad_shift.reshape(ctx.mod_shape).to(ctx.mod_dtype)
+        return grad_input, grad_scale, grad_shift, None, None
+
+
+class AdaLNCustom(nn.Module):
+    """Module form of AdaLNModelFunction (dit_fusedlayers.py:139-153)."""
+
+    def __init__(self, hidden_size, eps=1e-6):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.eps = eps
+
+    def forward(self, x, scale, shift):
+        cols = self.hidden_size
+        for name, t in (("input x", x), ("scale", scale), ("shift", shift)):
+            if t.shape[-1] != cols:
+                raise ValueError(f"Last dim of {name} must be hidden_size {cols}, got {t.shape[-1]}")
+        return AdaLNModelFunction.apply(x, scale, shift, self.eps, cols)
+
+
+def modulated_layer_norm(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6):
+    """LayerNorm(x) * (1 + scale[:, None]) + shift[:, None] through the fused kernel.
+
+    The same math as the adaLN-Zero input norm; also what the reference leaves
+    un-fused after attention (`norm2` + modulate, dit_layerspec.py:158-167) and
+    in the output head (AdaLNContinuous, dit_layerspec.py:55-78)."""
+    return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
+
+
+def _make_modulation_linear(embedding_dim: int, n_chunks: int, bias: bool, linear_parallel: bool, config):
+    if not linear_parallel:
+        return nn.Linear(embedding_dim, n_chunks * embedding_dim, bias=bias)
+    # The reference builds a Megatron/TransformerEngine column-parallel linear here
+    # (dit_fusedlayers.py:184-192); that stack is a dependency of the caller, not of this package.
+    assert config is not None
+    try:
+        from megatron.core.transformer.custom_layers.transformer_engine import TEColumnParallelLinear
+    except ImportError as exc:
+        raise ImportError("linear_parallel=True needs megatron.core's TEColumnParallelLinear; "
+                          "pass linear_parallel=False to use nn.Linear") from exc
+    return TEColumnParallelLinear(input_size=embedding_dim, output_size=n_chunks * embedding_dim, config=config,
+                                  gather_output=False, init_method=config.init_method, bias=bias,
+                                  skip_bias_add=False, is_expert=False)
+
+
+def _gather_modulation(emb, linear_parallel: bool):
+    if not linear_parallel:
+        return emb
+    from megatron.core.tensor_parallel.mappings import gather_from_tensor_model_parallel_region
+    return gather_from_tensor_model_parallel_region(emb[0])
+
+
+class _AdaLNZeroBase(nn.Module):
+    """Shared part of the two adaLN-Zero modules: SiLU -> linear -> chunks, then
+    the modulated LayerNorm, fused or eager as the constructor flag says."""
+
+    n_chunks = 0
+
+    def __init__(self, embedding_dim: int, norm_type: str, bias: bool, fused_kernels: bool,
+                 linear_parallel: bool, config):
+        super().__init__()
+        self.silu = nn.SiLU()
+        self.linear_parallel = linear_parallel
+        self.linear = _make_modulation_linear(embedding_dim, self.n_chunks, bias, linear_parallel, config)
+        self.fused_kernels = bool(fused_kernels)
+        self.embedding_dim = embedding_dim
+        if self.fused_kernels:
+            if embedding_dim not in SUPPORTED_COLS:
+                raise ValueError(f"fused_kernels=True needs embedding_dim in {SUPPORTED_COLS}, got {embedding_dim}")
+            _require_extension(fused_adaln, "fused_adaln")
+            self.adaLN = AdaLNCustom(embedding_dim, eps=1e-6)
+        elif norm_type == "layer_norm":
+            self.norm = nn.LayerNorm(embedding_dim, elementwise_affine=False, eps=1e-6)
+        elif norm_type == "fp32_layer_norm":
+            self.norm = FP32LayerNorm(embedding_dim, elementwise_affine=False, bias=False)
+        else:
+            raise ValueError(f"Unsupported `norm_type` ({norm_type}) provided. "
+                             "Supported ones are: 'layer_norm', 'fp32_layer_norm'.")
+
+    def _modulate(self, x, scale, shift):
+        if self.fused_kernels:
+            return self.adaLN(x, scale, shift)
+        return self.norm(x) * (1 + scale[:, None]) + shift[:, None]
+
+
+class FusedAdaLayerNormZero(_AdaLNZeroBase):
+    """adaLN-Zero for the double-stream blocks (dit_fusedlayers.py:155-224):
+    returns (x_mod, gate_msa, shift_mlp, scale_mlp, gate_mlp)."""
+
+    n_chunks = 6
+
+    def __init__(self, embedding_dim: int, num_embeddings: Optional[int] = None, norm_type="layer_norm",
+                 bias=True, fused_kernels=False, linear_parallel=True, config=None):
+        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config)
+        self.emb = None
+        if num_embeddings is not None:
+            try:
+                from diffusers.models.embeddings import CombinedTimestepLabelEmbeddings
+            except ImportError as exc:
+                raise ImportError("num_embeddings needs diffusers' CombinedTimestepLabelEmbeddings") from exc
+            self.emb = CombinedTimestepLabelEmbeddings(num_embeddings, embedding_dim)
+
+    def forward(self, x, timestep=None, class_labels=None, hidden_dtype=None, emb=None):
+        if self.emb is not None:
+            emb = self.emb(timestep, class_labels, hidden_dtype=hidden_dtype)
+        emb = _gather_modulation(self.linear(self.silu(emb)), self.linear_parallel)
+        shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = emb.chunk(6, dim=1)
+        return self._modulate(x, scale_msa, shift_msa), gate_msa, shift_mlp, scale_mlp, gate_mlp
+
+
+class FusedAdaLayerNormZeroSingle(_AdaLNZeroBase):
+    """adaLN-Zero for the single-stream blocks (dit_fusedlayers.py:226-272):
+    returns (x_mod, gate_msa)."""
+
+    n_chunks = 3
+
+    def __init__(self, embedding_dim: int, norm_type="layer_norm", bias=True, fused_kernels=False,
+                 linear_parallel=True, config=None):
+        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config)
+
+    def forward(self, x, emb=None):
+        emb = _gather_modulation(self.linear(self.silu(emb)), self.linear_parallel)
+        shift_msa, scale_msa, gate_msa = emb.chunk(3, dim=1)
+        return self._modulate(x, scale_msa, shift_msa), gate_msa
+
+
+class RMSNormModelFunction(Function):
+    """out = (x * rsqrt(mean(x^2) + eps)) * weight over the last `cols` elements.
+
+    apply(x, weight, epsilon, cols) -> out, with gradients for x and weight
+    (dit_fusedlayers.py:281,317)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, epsilon, cols):
+        ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
+        _require_gpu(x, "RMSNormModelFunction")
+        x = x.contiguous()
+        if cols not in SUPPORTED_COLS or x.numel() == 0 or x.numel() % cols != 0:
+            raise ValueError(f"Input size {x.numel()} not divisible by cols {cols} or unsupported cols value "
+                             f"(supported: {SUPPORTED_COLS})")
+        if weight.numel() != cols:
+            raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
+        w = weight.contiguous()
+        if w.dtype != x.dtype:
+            w = w.to(x.dtype)
+        rows = x.numel() // cols
+        out = torch.empty_like(x)
+        invvar = torch.empty(rows, device=x.device, dtype=torch.float32)
+        ext.torch_launch_rms_forward(out, x, w, rows, cols, float(epsilon), invvar)
+        ctx.save_for_backward(x, w, invvar)
+        ctx.rows, ctx.cols = rows, cols
+        ctx.w_shape, ctx.w_dtype = weight.shape, weight.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, w, invvar = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        if grad_output.dtype != x.dtype:
+            grad_output = grad_output.to(x.dtype)
+        grad_input = torch.empty_like(x)
+        grad_weight = torch.empty_like(w)
+        fused_rmsnorm.torch_launch_rms_backward_x(grad_input, grad_weight, grad_output, x, w, invvar,
+                                                  ctx.rows, ctx.cols)
+        return grad_input, grad_weight.reshape(ctx.w_shape).to(ctx.w_dtype), None, None
+
+
+class RMSNorm(nn.Module):
+    """RMSNorm with a learnable scale (dit_fusedlayers.py:353-370).  Uses the fused
+    kernel when FUSED_KERNELS is on and hidden_size is one the kernels are built
+    for; otherwise the reference's eager formula."""
+
+    def __init__(self, hidden_size: int, config=None, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.hidden_size = hidden_size
+
+    def _norm(self, x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
+
+    def forward(self, x):
+        if fused_kernels_requested() and self.hidden_size in SUPPORTED_COLS:
+            return RMSNormModelFunction.apply(x, self.weight, self.eps, self.hidden_size)
+        return self._norm(x.float()).type_as(x) * self.weight
+
+
+def Get_RMSNorm():
+    """Returns the RMSNorm class (the reference hands the class out through a
+    factory, dit_fusedlayers.py:350-375)."""
+    return RMSNorm
+
+
+def install_as_teletron_op() -> None:
+    """Registers the extension modules under the reference's top-level names so
+    that `import fused_adaln` / `import fused_rmsnorm` in unmodified reference
+    code (dit_fusedlayers.py:35-45) picks up this build."""
+    import sys
+    sys.modules.setdefault("fused_adaln", _require_extension(fused_adaln, "fused_adaln"))
+    sys.modules.setdefault("fused_rmsnorm", _require_extension(fused_rmsnorm, "fused_rmsnorm"))

@@ -1,0 +1,197 @@
+"""GPU tests of the operator interface: the autograd Functions and modules of
+teletron_amd.fusedlayers (the names HunyuanVideo blocks import), driven the way
+the reference's callers drive them, against the eager oracle.  Same bars as
+tests/test_gpu_parity.py."""
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+
+pytestmark = pytest.mark.gpu
+EPS = 1e-6
+
+
+@pytest.fixture(scope="module")
+def FL(gpu_device):
+    from teletron_amd import fusedlayers
+    assert fusedlayers.fused_kernels_available()
+    return fusedlayers
+
+
+def fwd_ok(got, want, excuse):
+    rep = O.compare_bf16_ulp(got.detach().cpu(), want, excuse_abs=excuse)
+    assert rep.n_gt1 == 0 and rep.n_excused <= 1e-4 * rep.n and rep.frac_exact >= 0.999, rep
+
+
+def grad_ok(got, want, allow=0.0):
+    assert got.shape == want.shape and got.dtype == want.dtype
+    assert O.frac_outside(got.cpu(), want, 1e-2, 1e-3) <= allow
+
+
+def test_adaln_function_autograd_per_sample(FL, gpu_device):
+    d = O.make_adaln_inputs(3, 257, 3072, torch.bfloat16, seed=41)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    x = d["x"].to(gpu_device).requires_grad_(True)
+    sc = d["scale"].to(gpu_device).requires_grad_(True)
+    sh = d["shift"].to(gpu_device).requires_grad_(True)
+    out = FL.AdaLNModelFunction.apply(x, sc, sh, EPS, 3072)
+    assert out.shape == x.shape and out.dtype == x.dtype
+    out.backward(d["grad"].to(gpu_device))
+    fwd_ok(out, want_out, O.adaln_excuse(d["x"], d["scale"], d["shift"], want_out))
+    grad_ok(x.grad, want_dx, allow=1e-5)
+    grad_ok(sc.grad, want_ds)
+    grad_ok(sh.grad, want_dh)
+
+
+def test_adaln_function_single_row_modulation_1d(FL, gpu_device):
+    """scale/shift given as [cols] (the shape the reference's docstring names)."""
+    d = O.make_adaln_inputs(1, 300, 3072, torch.bfloat16, seed=42)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    x = d["x"][0].to(gpu_device).requires_grad_(True)              # [S, C]
+    sc = d["scale"][0].to(gpu_device).requires_grad_(True)         # [C]
+    sh = d["shift"][0].to(gpu_device).requires_grad_(True)
+    out = FL.AdaLNModelFunction.apply(x, sc, sh, EPS, 3072)
+    out.backward(d["grad"][0].to(gpu_device))
+    fwd_ok(out, want_out[0], O.adaln_excuse(d["x"], d["scale"], d["shift"], want_out)[0])
+    grad_ok(sc.grad, want_ds[0])
+    grad_ok(sh.grad, want_dh[0])
+    grad_ok(x.grad, want_dx[0], allow=1e-5)
+
+
+def test_adaln_function_value_errors(FL, gpu_device):
+    x = torch.zeros(2, 4, 3072, dtype=torch.bfloat16, device=gpu_device)
+    m = torch.zeros(2, 3072, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(ValueError, match="cols"):
+        FL.AdaLNModelFunction.apply(x, m, m, EPS, 1024)
+    with pytest.raises(ValueError, match="modulation rows"):
+        FL.AdaLNModelFunction.apply(x, torch.zeros(4, 3072, dtype=torch.bfloat16, device=gpu_device),
+                                    torch.zeros(4, 3072, dtype=torch.bfloat16, device=gpu_device), EPS, 3072)
+    with pytest.raises(ValueError):
+        FL.RMSNormModelFunction.apply(x, torch.ones(3072, device=gpu_device), EPS, 1000)
+
+
+def test_rmsnorm_function_on_transposed_qk(FL, gpu_device):
+    """The attention caller normalises query.transpose(1, 2): [B, H, S, D], non-contiguous
+    (dit_attention.py:201-212)."""
+    B, S, H, D = 2, 300, 24, 128
+    d = O.make_rmsnorm_inputs((B, S, H), D, torch.bfloat16, seed=43)
+    xt = d["x"].transpose(1, 2)                                    # [B, H, S, D] view
+    gt = d["grad"].transpose(1, 2).contiguous()
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(xt, d["weight"], gt)
+    x = d["x"].to(gpu_device).requires_grad_(True)
+    w = d["weight"].to(gpu_device).requires_grad_(True)
+    out = FL.RMSNormModelFunction.apply(x.transpose(1, 2), w, EPS, D)
+    assert out.shape == (B, H, S, D)
+    out.backward(gt.to(gpu_device))
+    fwd_ok(out, want_out, O.rmsnorm_excuse(want_out))
+    grad_ok(w.grad, want_dw)
+    grad_ok(x.grad, want_dx.transpose(1, 2))                       # want_dx is w.r.t. the transposed view
+
+
+def test_rmsnorm_module_fused_branch(FL, gpu_device, monkeypatch):
+    monkeypatch.setenv("FUSED_KERNELS", "1")
+    for cols in (128, 3072):
+        d = O.make_rmsnorm_inputs((4, 50), cols, torch.bfloat16, seed=44)
+        want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+        m = FL.Get_RMSNorm()(cols, config=None).to(gpu_device).bfloat16()
+        with torch.no_grad():
+            m.weight.copy_(d["weight"])
+        x = d["x"].to(gpu_device).requires_grad_(True)
+        out = m(x)
+        out.backward(d["grad"].to(gpu_device))
+        fwd_ok(out, want_out, O.rmsnorm_excuse(want_out))
+        grad_ok(x.grad, want_dx)
+        grad_ok(m.weight.grad, want_dw)
+    monkeypatch.setenv("FUSED_KERNELS", "0")                       # eager branch on the GPU: same module
+    out_eager = m(x)
+    assert O.compare_bf16_ulp(out_eager.detach().cpu(), want_out).n_gt1 == 0
+
+
+def test_rmsnorm_function_fp32_weight_with_bf16_input(FL, gpu_device):
+    """An uncast fp32 parameter is rounded to the activation dtype; its gradient comes back fp32."""
+    d = O.make_rmsnorm_inputs((64,), 128, torch.bfloat16, seed=45)
+    x = d["x"].to(gpu_device).requires_grad_(True)
+    w32 = d["weight"].float().to(gpu_device).requires_grad_(True)
+    out = FL.RMSNormModelFunction.apply(x, w32, EPS, 128)
+    out.backward(d["grad"].to(gpu_device))
+    assert out.dtype == torch.bfloat16 and w32.grad.dtype == torch.float32 and w32.grad.shape == (128,)
+    want_out, _, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    fwd_ok(out, want_out, O.rmsnorm_excuse(want_out))
+    assert O.frac_outside(w32.grad.cpu(), want_dw.float(), 1e-2, 1e-3) == 0.0
+
+
+def test_adaln_zero_modules_fused_vs_eager_branch(FL, gpu_device):
+    """FusedAdaLayerNormZero / ...Single with fused_kernels on and off share weights and
+    must agree (hidden 3072, per-sample temb), forward and backward."""
+    torch.manual_seed(0)
+    B, S, C = 2, 130, 3072
+    x = torch.randn(B, S, C, device=gpu_device).bfloat16()
+    temb = torch.randn(B, C, device=gpu_device).bfloat16()
+    g = torch.randn(B, S, C, device=gpu_device).bfloat16()
+    for cls in (FL.FusedAdaLayerNormZero, FL.FusedAdaLayerNormZeroSingle):
+        fused = cls(C, fused_kernels=True, linear_parallel=False).to(gpu_device).bfloat16()
+        eager = cls(C, fused_kernels=False, linear_parallel=False).to(gpu_device).bfloat16()
+        eager.load_state_dict(fused.state_dict())
+        xa = x.clone().requires_grad_(True)
+        xb = x.clone().requires_grad_(True)
+        ya = fused(xa, emb=temb)
+        yb = eager(xb, emb=temb)
+        assert len(ya) == len(yb) == (5 if cls is FL.FusedAdaLayerNormZero else 2)
+        for a, b in zip(ya[1:], yb[1:]):
+            assert torch.equal(a, b)                                # gates / mlp modulation pass through
+        ya[0].backward(g)
+        yb[0].backward(g)
+        rep = O.compare_bf16_ulp(ya[0].detach().cpu(), yb[0].detach().cpu())
+        assert rep.frac_exact > 0.999
+        assert O.frac_outside(ya[0].detach().cpu(), yb[0].detach().cpu(), 1e-2, 1e-3) < 1e-5
+        assert O.frac_outside(xa.grad.cpu(), xb.grad.cpu(), 1e-2, 1e-3) < 1e-5
+        # the modulation linear receives dscale/dshift: weight grads agree to bf16 accumulation noise
+        ga, gb = fused.linear.weight.grad.float().cpu(), eager.linear.weight.grad.float().cpu()
+        assert (ga - gb).abs().max() <= 2e-2 * gb.abs().max()
+
+
+def test_modulated_layer_norm_matches_unfused_norm2_site(FL, gpu_device):
+    """norm2 + modulate as written in the double-stream block (dit_layerspec.py:158-167)."""
+    d = O.make_adaln_inputs(2, 200, 3072, torch.bfloat16, seed=46)
+    ln = torch.nn.LayerNorm(3072, elementwise_affine=False, eps=1e-6)
+    want = ln(d["x"]) * (1 + d["scale"][:, None]) + d["shift"][:, None]
+    got = FL.modulated_layer_norm(d["x"].to(gpu_device), d["scale"].to(gpu_device), d["shift"].to(gpu_device))
+    fwd_ok(got, want, O.adaln_excuse(d["x"], d["scale"], d["shift"], want))
+
+
+def test_reference_signature_extension_calls(FL, gpu_device):
+    """Drive the extension exactly as the reference's autograd classes do
+    (dit_fusedlayers.py:95-104,128-136,305-313,337-346)."""
+    d = O.make_adaln_inputs(1, 333, 3072, torch.bfloat16, seed=47)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    x, scale, shift, grad = (d[k].to(gpu_device) for k in ("x", "scale", "shift", "grad"))
+    rows, cols = 333, 3072
+    output, x_norm = torch.empty_like(x), torch.empty_like(x)
+    invvar = torch.empty(rows, device=gpu_device, dtype=torch.float32)
+    FL.fused_adaln.torch_launch_adaln_forward(output, x_norm, x, scale, shift, rows, cols, EPS, invvar)
+    grad_input, grad_scale, grad_shift = torch.empty_like(x_norm), torch.empty_like(scale), torch.empty_like(scale)
+    FL.fused_adaln.torch_launch_adaln_backward(grad_input, grad_scale, grad_shift, grad, x_norm, scale, invvar,
+                                               rows, cols)
+    fwd_ok(output, want_out, O.adaln_excuse(d["x"], d["scale"], d["shift"], want_out))
+    assert O.frac_outside(grad_input.cpu(), want_dx, 1e-2, 1e-3) < 1e-3
+    grad_ok(grad_scale, want_ds)
+    grad_ok(grad_shift, want_dh)
+
+    r = O.make_rmsnorm_inputs((1, 400, 24), 128, torch.bfloat16, seed=48)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(r["x"], r["weight"], r["grad"])
+    x, w, grad = (r[k].to(gpu_device) for k in ("x", "weight", "grad"))
+    rows = x.numel() // 128
+    output = torch.empty_like(x)
+    invvar = torch.empty(rows, device=gpu_device, dtype=torch.float32)
+    FL.fused_rmsnorm.torch_launch_rms_forward(output, x, w, rows, 128, EPS, invvar)
+    grad_input, grad_weight = torch.empty_like(output), torch.empty_like(w)
+    FL.fused_rmsnorm.torch_launch_rms_backward(grad_input, grad_weight, grad, output, w, invvar, rows, 128)
+    fwd_ok(output, want_out, O.rmsnorm_excuse(want_out))
+    assert O.frac_outside(grad_input.cpu(), want_dx, 1e-2, 1e-3) < 1e-3
+    assert O.frac_outside(grad_weight.cpu(), want_dw, 3e-2, 1e-1) == 0.0
+    # registered operator form
+    out2 = torch.empty_like(x)
+    torch.ops.Fused_RMSNorm.torch_launch_rms_forward(out2, x, w, rows, 128, EPS, invvar)
+    assert torch.equal(out2, output)
+    with pytest.raises(RuntimeError, match="elements"):
+        FL.fused_rmsnorm.torch_launch_rms_forward(output, x, w, rows + 1, 128, EPS, invvar)

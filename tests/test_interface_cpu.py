@@ -1,0 +1,140 @@
+"""CPU-side checks of the boundary: the C ABI library exports what the header
+declares, the extension modules expose the reference's function names, host
+argument checking works, and the module-level selection logic follows the
+reference (eager math when FUSED_KERNELS is off).  No kernel is launched."""
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "teletron_norm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tt_\w+)\s*\(", text)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    from teletron_amd import capi
+    L = capi.lib()
+    names = _declared_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in teletron_norm.h but not exported"
+    assert sorted(capi.EXPORTS) == names
+    assert L.tt_norm_abi_version() == 1
+    assert L.tt_norm_status_string(0) == b"ok"
+    assert L.tt_norm_status_string(4).startswith(b"workspace")
+    assert L.tt_norm_supported(3072, capi.BF16) == 1 and L.tt_norm_supported(128, capi.F32) == 1
+    assert L.tt_norm_supported(1024, capi.BF16) == 0 and L.tt_norm_supported(3072, 5) == 0
+
+
+def test_c_abi_argument_errors_need_no_gpu():
+    from teletron_amd import capi
+    L = capi.lib()
+    assert L.tt_rmsnorm_forward(None, None, None, None, 4, 3072, 1e-6, 0, None) == 1      # null pointers
+    assert L.tt_rmsnorm_forward(None, None, None, None, 4, 1000, 1e-6, 0, None) == 2      # unsupported cols
+    assert b"cols=1000" in L.tt_norm_last_error()
+    assert L.tt_adaln_forward(None, None, None, None, None, None, 0, 4, 3072, 1e-6, 0, None) == 1
+    assert L.tt_norm_stream_copy(None, None, 32, None) == 1
+
+
+def test_extension_modules_expose_reference_names():
+    from teletron_amd import fusedlayers as FL
+    assert FL.fused_kernels_available()
+    for fn in ("torch_launch_rms_forward", "torch_launch_rms_backward", "torch_launch_rms_backward_x"):
+        assert callable(getattr(FL.fused_rmsnorm, fn))
+    for fn in ("torch_launch_adaln_forward", "torch_launch_adaln_backward",
+               "torch_launch_adaln_forward_stats", "torch_launch_adaln_backward_x"):
+        assert callable(getattr(FL.fused_adaln, fn))
+    # operator-library registrations under the reference's namespaces
+    assert hasattr(torch.ops.Fused_RMSNorm, "torch_launch_rms_forward")
+    assert hasattr(torch.ops.layernorm_block_smem, "torch_launch_adaln_backward")
+    FL.install_as_teletron_op()
+    import fused_adaln
+    import fused_rmsnorm
+    assert fused_adaln is FL.fused_adaln and fused_rmsnorm is FL.fused_rmsnorm
+
+
+def test_extension_rejects_cpu_tensors_loudly():
+    from teletron_amd import fusedlayers as FL
+    x = torch.zeros(2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        FL.fused_rmsnorm.torch_launch_rms_forward(torch.empty_like(x), x, torch.ones(128, dtype=torch.bfloat16),
+                                                  2, 128, 1e-6, torch.empty(2))
+    with pytest.raises(ValueError, match="GPU tensor"):
+        FL.RMSNormModelFunction.apply(x, torch.ones(128, dtype=torch.bfloat16), 1e-6, 128)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        FL.AdaLNModelFunction.apply(torch.zeros(1, 2, 3072), torch.zeros(1, 3072), torch.zeros(1, 3072), 1e-6, 3072)
+
+
+def test_adaln_custom_shape_errors():
+    from teletron_amd import fusedlayers as FL
+    m = FL.AdaLNCustom(3072)
+    with pytest.raises(ValueError, match="input x"):
+        m(torch.zeros(1, 2, 128), torch.zeros(1, 3072), torch.zeros(1, 3072))
+    with pytest.raises(ValueError, match="scale"):
+        m(torch.zeros(1, 2, 3072), torch.zeros(1, 128), torch.zeros(1, 3072))
+    with pytest.raises(ValueError, match="shift"):
+        m(torch.zeros(1, 2, 3072), torch.zeros(1, 3072), torch.zeros(1, 128))
+
+
+def test_rmsnorm_module_env_gate_and_eager_branch(monkeypatch):
+    from teletron_amd import fusedlayers as FL
+    RMSNorm = FL.Get_RMSNorm()
+    assert RMSNorm is FL.RMSNorm
+    m = RMSNorm(128, config=None)
+    assert m.weight.shape == (128,) and m.eps == 1e-6 and m.hidden_size == 128
+    d = O.make_rmsnorm_inputs((5, 7), 128, torch.bfloat16, seed=1)
+    with torch.no_grad():
+        m.weight.copy_(d["weight"].float())
+    m = m.bfloat16()
+    monkeypatch.delenv("FUSED_KERNELS", raising=False)
+    assert not FL.fused_kernels_requested()
+    assert torch.equal(m(d["x"]), O.eager_rmsnorm(d["x"], d["weight"]))
+    monkeypatch.setenv("FUSED_KERNELS", "0")
+    assert not FL.fused_kernels_requested()
+    assert torch.equal(m(d["x"]), O.eager_rmsnorm(d["x"], d["weight"]))
+    monkeypatch.setenv("FUSED_KERNELS", "1")
+    assert FL.fused_kernels_requested()
+    with pytest.raises(ValueError, match="GPU tensor"):   # fused requested: no quiet CPU fallback
+        m(d["x"])
+    other = RMSNorm(96, config=None)                        # a width the kernels are not built for
+    assert other(torch.ones(2, 96)).shape == (2, 96)
+
+
+def test_adaln_zero_modules_eager_branch_matches_oracle():
+    from teletron_amd import fusedlayers as FL
+    torch.manual_seed(0)
+    B, S, C = 2, 5, 64
+    x = torch.randn(B, S, C)
+    temb = torch.randn(B, C)
+    m6 = FL.FusedAdaLayerNormZero(C, linear_parallel=False)
+    out, gate_msa, shift_mlp, scale_mlp, gate_mlp = m6(x, emb=temb)
+    chunks = m6.linear(torch.nn.functional.silu(temb)).chunk(6, dim=1)
+    torch.testing.assert_close(out, O.eager_adaln(x, chunks[1], chunks[0]))
+    for got, want in zip((gate_msa, shift_mlp, scale_mlp, gate_mlp), chunks[2:]):
+        assert torch.equal(got, want)
+    m3 = FL.FusedAdaLayerNormZeroSingle(C, linear_parallel=False, norm_type="fp32_layer_norm")
+    out3, gate3 = m3(x, emb=temb)
+    c3 = m3.linear(torch.nn.functional.silu(temb)).chunk(3, dim=1)
+    # the reference builds FP32LayerNorm without eps, i.e. with nn.LayerNorm's default 1e-5
+    torch.testing.assert_close(out3, O.eager_adaln(x, c3[1], c3[0], eps=1e-5))
+    assert torch.equal(gate3, c3[2])
+    with pytest.raises(ValueError, match="norm_type"):
+        FL.FusedAdaLayerNormZeroSingle(C, linear_parallel=False, norm_type="nope")
+    with pytest.raises(ValueError, match="embedding_dim"):
+        FL.FusedAdaLayerNormZero(C, linear_parallel=False, fused_kernels=True)
+
+
+def test_fp32_layer_norm():
+    from teletron_amd import fusedlayers as FL
+    x = torch.randn(3, 64, generator=torch.Generator().manual_seed(0)).bfloat16()
+    ln = FL.FP32LayerNorm(64, elementwise_affine=False, bias=False)
+    want = torch.nn.functional.layer_norm(x.float(), (64,), None, None, ln.eps).bfloat16()
+    assert torch.equal(ln(x), want)
