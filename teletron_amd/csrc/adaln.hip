@@ -121,26 +121,39 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     }
 }
 
-// FROM_XNORM = false: xin is the saved input x, statistics mean/rstd.
-// FROM_XNORM = true : xin is the saved normalised row rnd(LN(x)); only rstd is used.
+// Backward.  FROM_XNORM = false: xin is the saved input x, statistics mean/rstd.
+//            FROM_XNORM = true : xin is the saved normalised row rnd(LN(x)); only rstd is used.
+//
+// Same structure as the RMSNorm backward: one wavefront per SIMD at 3072
+// columns, modulation row unpacked once, column sums in registers, next row in
+// flight while the current one is processed.  With xhat = x*r - mu*r the row
+// reductions reduce to sum_c gx and sum_c gx*x, both taken straight from packed
+// bf16 pairs, and dx becomes r*gx + x*K1 + K0 with per-row scalars K1, K0.
 template <typename T, int C, bool FROM_XNORM>
-__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void adaln_bwd_kernel(
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 : 4) void adaln_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
     const float *__restrict__ rstd, int64_t rows_per_sample, int blocks_per_sample) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    // fp32 rows of 3072 need 96 registers per row buffer: no room for a second one
+    constexpr bool kDoubleBuffer = !(sizeof(T) == 4 && C >= 1024);
     __shared__ float lds[2 * C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
     const int l = lane % LANES;
     const int wave = wave_id_in_block();
-    const int64_t b = blockIdx.x / blocks_per_sample;
+    const int64_t smp = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
 
-    u32x4 tr[CHUNKS];
-    load_one_plus_scale<T, C>(tr, scale + b * C, l);
+    float tv[CHUNKS][VEC];  // t = rnd(1 + scale[sample]), unpacked once
+    {
+        u32x4 tr[CHUNKS];
+        load_one_plus_scale<T, C>(tr, scale + smp * C, l);
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) E::unpack(tr[k], tv[k]);
+    }
 
     float acc[2][CHUNKS][VEC];  // [0] = dscale, [1] = dshift
 #pragma unroll
@@ -150,67 +163,80 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[s][k][j] = 0.0f;
 
-    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
-    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
-    for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
-        keep_packed(tr);
-        const int64_t rs = grp * RPW + sub;
-        const bool ok = rs < rows_per_sample;
-        const int64_t row = b * rows_per_sample + rs;
-        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + row * C) + l;
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + row * C) + l;
-        u32x4 gr[CHUNKS], xr[CHUNKS];
+    struct RowRegs {
+        u32x4 g[CHUNKS], x[CHUNKS];
+        float r, mu;
+        int64_t row;
+        bool ok;
+    };
+    auto fetch = [&](RowRegs &b, int64_t grp) {
+        const int64_t rs = grp * RPW + sub;  // row inside the sample
+        b.ok = rs < rows_per_sample;
+        b.row = smp * rows_per_sample + rs;
+        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            gr[k] = ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
-            xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+            b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+            b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
-        const float r = ok ? rstd[row] : 0.0f;
-        const float mu = (!FROM_XNORM && ok) ? mean[row] : 0.0f;
-
+        b.r = b.ok ? rstd[b.row] : 0.0f;
+        b.mu = (!FROM_XNORM && b.ok) ? mean[b.row] : 0.0f;
+    };
+    auto process = [&](const RowRegs &b) {
+        const float r = b.r, mu = b.mu;
+        const float nmr = -(mu * r);  // xhat = x*r + nmr
+        // pass 1: gx = rnd(g*t) kept packed; s1 = sum_c gx; s2 = sum_c gx * xhat
+        u32x4 gxp[CHUNKS];
         float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], xv[VEC], tv[VEC];
-            E::unpack(gr[k], gv);
-            E::unpack(xr[k], xv);
-            E::unpack(tr[k], tv);
+            float gv[VEC];
+            E::unpack(b.g[k], gv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) gv[j] *= tv[j];
-            E::round(gv);  // gx materialised in the element type
+            for (int j = 0; j < VEC; ++j) gv[j] *= tv[k][j];
+            gxp[k] = E::pack(gv);  // gx materialised in the element type
+            if constexpr (kIsBf16<T>) {
+                // s2 accumulates sum_c gx * xin here; turned into sum_c gx * xhat below
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                const float xh = FROM_XNORM ? xv[j] : (xv[j] - mu) * r;
-                s1 += gv[j];
-                s2 = fmaf(gv[j], xh, s2);
+                for (int i = 0; i < 4; ++i) {
+                    s1 = dot2_bf16(gxp[k][i], kBf16OnesPair, s1);
+                    s2 = dot2_bf16(gxp[k][i], b.x[k][i], s2);
+                }
+            } else {
+                float gx[VEC], xv[VEC];
+                E::unpack(gxp[k], gx);
+                E::unpack(b.x[k], xv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    s1 += gx[j];
+                    s2 = fmaf(gx[j], FROM_XNORM ? xv[j] : fmaf(xv[j], r, nmr), s2);
+                }
             }
         }
-        const float m1 = group_sum<LANES>(s1) / (float)C;
-        const float m2 = group_sum<LANES>(s2) / (float)C;
-        const float k0 = -(r * m1), k1 = -(r * m2);  // dx = r*gx + xhat*k1 + k0
-        // Pass 2 re-derives gx and xhat from the packed registers instead of keeping
-        // them live across the reductions (registers buy occupancy here).
-        keep_packed(gr);
-        keep_packed(xr);
+        s1 = group_sum<LANES>(s1);
+        s2 = group_sum<LANES>(s2);
+        if constexpr (kIsBf16<T> && !FROM_XNORM) s2 = r * (s2 - mu * s1);
+        const float m1 = s1 / (float)C, m2 = s2 / (float)C;
+        // dx = r*gx + xhat*k1 + k0,  k1 = -r*m2, k0 = -r*m1;  in terms of xin: r*gx + xin*K1 + K0
+        const float k1 = -(r * m2), k0 = -(r * m1);
+        const float K1 = FROM_XNORM ? k1 : k1 * r;
+        const float K0 = FROM_XNORM ? k0 : fmaf(k1, nmr, k0);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.row * C) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], gx[VEC], xv[VEC], tv[VEC], o[VEC], xn[VEC];
-            E::unpack(gr[k], gv);
-            E::unpack(xr[k], xv);
-            E::unpack(tr[k], tv);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) gx[j] = gv[j] * tv[j];
-            E::round(gx);
+            float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
+            E::unpack(b.g[k], gv);
+            E::unpack(gxp[k], gx);
+            E::unpack(b.x[k], xv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                const float xh = FROM_XNORM ? xv[j] : (xv[j] - mu) * r;
-                o[j] = fmaf(r, gx[j], fmaf(xh, k1, k0));
-                xn[j] = xh;
+                o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
+                xn[j] = FROM_XNORM ? xv[j] : fmaf(xv[j], r, nmr);
                 acc[1][k][j] += gv[j];
             }
-            if (ok) store16_stream(pd + k * LANES, E::pack(o));
+            if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
             if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
@@ -218,14 +244,51 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[0][k][j] += xn[j];
         }
+    };
+
+    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
+    int64_t grp = (int64_t)slot * kRowWaves + wave;
+    if constexpr (kDoubleBuffer) {
+        if (grp < groups) {
+            RowRegs a, b;
+            fetch(a, grp);
+            for (;;) {
+                int64_t nxt = grp + stride;
+                bool more = nxt < groups;
+                if (more) fetch(b, nxt);
+                process(a);
+                if (!more) break;
+                grp = nxt + stride;
+                more = grp < groups;
+                if (more) fetch(a, grp);
+                process(b);
+                if (!more) break;
+            }
+        }
+    } else {
+        for (; grp < groups; grp += stride) {
+            RowRegs a;
+            fetch(a, grp);
+            process(a);
+        }
     }
     flush_column_partials<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds);
 }
 
+// Same launch policy as RMSNorm: forward one-shot at 3072 columns, backward one
+// workgroup per compute unit.
+constexpr int kOneShotGrid = 1 << 20;
+#ifndef TTN_ADALN_FWD_BLOCKS_PER_CU
+#define TTN_ADALN_FWD_BLOCKS_PER_CU (C >= 1024 ? kOneShotGrid : 16)
+#endif
+#ifndef TTN_ADALN_BWD_BLOCKS_PER_CU
+#define TTN_ADALN_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 4)
+#endif
 template <typename T, int C>
 struct AdalnTune {
-    static constexpr int kFwdBlocksPerCu = 8;
-    static constexpr int kBwdBlocksPerCu = 2;
+    static constexpr int kFwdBlocksPerCu = TTN_ADALN_FWD_BLOCKS_PER_CU;
+    static constexpr int kBwdBlocksPerCu = TTN_ADALN_BWD_BLOCKS_PER_CU;
 };
 
 struct AdalnArgs {

@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace ttn {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -45,6 +47,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     v[0] = (__bf16)lo;
     v[1] = (__bf16)hi;
     return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename T>
+inline constexpr bool kIsBf16 = std::is_same<T, bf16_t>::value;
+
+constexpr uint32_t kBf16OnesPair = 0x3F803F80u;  // (1.0, 1.0) as two bf16
+
+// acc + a.lo*b.lo + a.hi*b.hi over one dword of two bf16 each (v_dot2c_f32_bf16):
+// products of bf16 pairs are exact in fp32, so this is a row reduction step
+// taken straight from the packed registers, with no unpacking.
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
+                                           false);
 }
 
 template <typename T>

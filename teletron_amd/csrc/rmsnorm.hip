@@ -69,25 +69,42 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     }
 }
 
-// FROM_OUT = false: xin is the saved input x.
-// FROM_OUT = true : xin is the saved forward output; xhat is recovered as out/w.
+// Backward.  FROM_OUT = false: xin is the saved input x.
+//            FROM_OUT = true : xin is the saved forward output; xhat is recovered as out/w.
+//
+// One wavefront per SIMD at 3072 columns: the kernel is given the whole register
+// file so that the weight stays unpacked, the column sums stay in registers and
+// the NEXT row's g and x are already in flight while the current row is
+// processed (two row buffers, ping-pong).  Few, fat, always-loading wavefronts
+// keep about 48 KiB of reads in flight per compute unit, which is where this
+// memory system streams best; more resident wavefronts only add queueing.
 template <typename T, int C, bool FROM_OUT>
-__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 2 : 1) void rmsnorm_bwd_kernel(
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 : 4) void rmsnorm_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ w, const float *__restrict__ rstd,
     int64_t rows) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
+    constexpr bool kPackedDot = kIsBf16<T> && !FROM_OUT;  // sum_c gy*x straight from bf16 pairs
+    // fp32 rows of 3072 need 96 registers per row buffer: no room for a second one
+    constexpr bool kDoubleBuffer = !(sizeof(T) == 4 && C >= 1024);
     __shared__ float lds[C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
     const int l = lane % LANES;
     const int wave = wave_id_in_block();
 
-    u32x4 wr[CHUNKS];
+    float wv[CHUNKS][VEC];                     // weight, unpacked once
+    [[maybe_unused]] float winv[CHUNKS][VEC];  // 1/weight for the saved-output variant
 #pragma unroll
-    for (int k = 0; k < CHUNKS; ++k) wr[k] = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
+    for (int k = 0; k < CHUNKS; ++k) {
+        E::unpack(load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l), wv[k]);
+        if constexpr (FROM_OUT) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) winv[k][j] = __builtin_amdgcn_rcpf(wv[k][j]);
+        }
+    }
 
     float acc[1][CHUNKS][VEC];
 #pragma unroll
@@ -95,65 +112,66 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[0][k][j] = 0.0f;
 
-    const int64_t groups = (rows + RPW - 1) / RPW;
-    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
-    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
-        keep_packed(wr);
-        const int64_t row = grp * RPW + sub;
-        const bool ok = row < rows;
-        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + row * C) + l;
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + row * C) + l;
-        u32x4 gr[CHUNKS], xr[CHUNKS];
+    struct RowRegs {
+        u32x4 g[CHUNKS], x[CHUNKS];
+        float r;
+        int64_t row;
+        bool ok;
+    };
+    auto fetch = [&](RowRegs &b, int64_t grp) {
+        b.row = grp * RPW + sub;
+        b.ok = b.row < rows;
+        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            gr[k] = ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
-            xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+            b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+            b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
-        const float r = ok ? rstd[row] : 0.0f;
-
-        // pass 1 over registers: row dot product  sum_c gy * xs
+        b.r = b.ok ? rstd[b.row] : 0.0f;
+    };
+    auto process = [&](const RowRegs &b) {
+        const float r = b.r;
+        // pass 1: gy = rnd(g*w), kept packed in the element type; row dot  sum_c gy * xs
         //   xs = x (native) or xhat = out / w (from the saved output)
+        u32x4 gyp[CHUNKS];
         float dot = 0.0f;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], xv[VEC], wv[VEC];
-            E::unpack(gr[k], gv);
-            E::unpack(xr[k], xv);
-            E::unpack(wr[k], wv);
+            float gv[VEC];
+            E::unpack(b.g[k], gv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) gv[j] *= wv[j];
-            E::round(gv);  // gy materialised in the element type
+            for (int j = 0; j < VEC; ++j) gv[j] *= wv[k][j];
+            gyp[k] = E::pack(gv);  // gy materialised in the element type
+            if constexpr (kPackedDot) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-                const float xs = FROM_OUT ? xv[j] * __builtin_amdgcn_rcpf(wv[j]) : xv[j];
-                dot = fmaf(gv[j], xs, dot);
+                for (int i = 0; i < 4; ++i) dot = dot2_bf16(gyp[k][i], b.x[k][i], dot);
+            } else {
+                float gy[VEC], xv[VEC];
+                E::unpack(gyp[k], gy);
+                E::unpack(b.x[k], xv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) dot = fmaf(gy[j], FROM_OUT ? xv[j] * winv[k][j] : xv[j], dot);
             }
         }
         dot = group_sum<LANES>(dot);
-        // Pass 2 re-derives gy from the packed registers instead of keeping 2*C/LANES
-        // fp32 values live across the reduction (registers buy occupancy here).
-        keep_packed(gr);
-        keep_packed(xr);
         // dx = gy*r + xs*coef
         const float coef = FROM_OUT ? -(r * (dot / (float)C)) : -((dot / (float)C) * r * r * r);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.row * C) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], gy[VEC], xv[VEC], wv[VEC], o[VEC], y[VEC];
-            E::unpack(gr[k], gv);
-            E::unpack(xr[k], xv);
-            E::unpack(wr[k], wv);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) gy[j] = gv[j] * wv[j];
-            E::round(gy);
+            float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
+            E::unpack(b.g[k], gv);
+            E::unpack(gyp[k], gy);
+            E::unpack(b.x[k], xv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                const float xs = FROM_OUT ? xv[j] * __builtin_amdgcn_rcpf(wv[j]) : xv[j];
+                const float xs = FROM_OUT ? xv[j] * winv[k][j] : xv[j];
                 o[j] = fmaf(xs, coef, gy[j] * r);
                 y[j] = FROM_OUT ? xs : xs * r;
             }
-            if (ok) store16_stream(pd + k * LANES, E::pack(o));
+            if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
             E::round(y);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
@@ -161,15 +179,55 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[0][k][j] += y[j];
         }
+    };
+
+    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave;
+    if constexpr (kDoubleBuffer) {
+        if (grp < groups) {
+            RowRegs a, b;
+            fetch(a, grp);
+            for (;;) {
+                int64_t nxt = grp + stride;
+                bool more = nxt < groups;
+                if (more) fetch(b, nxt);
+                process(a);
+                if (!more) break;
+                grp = nxt + stride;
+                more = grp < groups;
+                if (more) fetch(a, grp);
+                process(b);
+                if (!more) break;
+            }
+        }
+    } else {
+        for (; grp < groups; grp += stride) {
+            RowRegs a;
+            fetch(a, grp);
+            process(a);
+        }
     }
     flush_column_partials<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds);
 }
 
 // ---- tuning: workgroups per compute unit of the persistent grids ------------
+// Forward at 3072 columns runs one-shot (one row per wavefront, then exit; the
+// hardware dispatcher keeps a steady mix of loading and storing wavefronts, which
+// streams ~6 % faster here than any persistent loop).  Forward at 128 columns and
+// both backward kernels are persistent; backward at 3072 columns uses one
+// workgroup per compute unit (one wavefront per SIMD).
+constexpr int kOneShot = 1 << 20;
+#ifndef TTN_RMS_FWD_BLOCKS_PER_CU
+#define TTN_RMS_FWD_BLOCKS_PER_CU (C >= 1024 ? kOneShot : 16)
+#endif
+#ifndef TTN_RMS_BWD_BLOCKS_PER_CU
+#define TTN_RMS_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 4)
+#endif
 template <typename T, int C>
 struct RmsTune {
-    static constexpr int kFwdBlocksPerCu = 8;
-    static constexpr int kBwdBlocksPerCu = 4;
+    static constexpr int kFwdBlocksPerCu = TTN_RMS_FWD_BLOCKS_PER_CU;
+    static constexpr int kBwdBlocksPerCu = TTN_RMS_BWD_BLOCKS_PER_CU;
 };
 
 template <typename T, int C>

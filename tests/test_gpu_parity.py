@@ -281,14 +281,14 @@ def test_batched_per_sample_modulation_chain(capi, gpu_device):
     assert rep.frac_exact > 0.995 and O.frac_outside(z_g.cpu(), z.detach(), 1e-2, 1e-3) < 1e-5
     dy, dw = capi.rmsnorm_backward(g["grad"], y_g, wg, rstd2)
     dx, ds, dh = capi.adaln_backward(dy, g["x"], g["scale"], mean, rstd)
-    # dweight sums 44 224 rows whose inputs (AdaLN outputs) already differ from eager's by the
-    # occasional one-ulp flip: columns whose sum nearly cancels can miss the absolute part of the
-    # bar; they must stay within 5x of it
-    assert_grad_bf16(dw, wr.grad, "dweight", allow=3e-3)
-    assert O.frac_outside(dw.cpu(), wr.grad, 5e-2, 5e-3) == 0.0
+    # The reduced gradients sum 11 056 (dscale, dshift) or 44 224 (dweight) rows whose inputs are
+    # the previous op's outputs, which already differ from eager's by the occasional one-ulp flip;
+    # a column whose sum nearly cancels can then miss the absolute part of the bar.  Such columns
+    # must be few and stay within 5x of it.
+    for name, got, want in (("dweight", dw, wr.grad), ("dscale", ds, sc.grad), ("dshift", dh, sh.grad)):
+        assert_grad_bf16(got, want, name, allow=3e-3)
+        assert O.frac_outside(got.cpu(), want, 5e-2, 5e-3) == 0.0, name
     assert_grad_bf16(dx, xr.grad, "dx", allow=1e-4)
-    assert_grad_bf16(ds, sc.grad, "dscale")
-    assert_grad_bf16(dh, sh.grad, "dshift")
 
 
 # ---------------------------------------------------------------- boundary
