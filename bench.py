@@ -29,7 +29,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (scaled by the same counters on the plain copy kernel); None until measured.
 MEASURED_TRAFFIC_BYTES = {
-    "adaln_backward": None,
+    # (FETCH_SIZE KiB * 2.000 + WRITE_SIZE KiB * 1.000) * 1024, see profiles/bench_cfg4_all_kernels.md
+    "rmsnorm_backward": int((714794.9 * 2.0 + 715872.2) * 1024),
+    "adaln_backward": int((716693.6 * 2.0 + 718944.0) * 1024),
+    "rmsnorm_forward": int((356452.9 * 2.0 + 713728.5) * 1024),
+    "adaln_forward": int((356497.4 * 2.0 + 714656.3) * 1024),
 }
 
 
