@@ -82,7 +82,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
-              "(rows shard trivially across GPUs; see DESIGN.md)", file=sys.stderr)
+              "(rows shard trivially across GPUs; nothing here uses a second one)", file=sys.stderr)
         sys.exit(2)
 
     import torch

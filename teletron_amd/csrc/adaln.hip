@@ -17,6 +17,18 @@
 #include "norm_device.h"
 #include "norm_host.h"
 
+// Backward pipeline shape at 3072 columns (measured back-to-back at 118 800 rows):
+// plain loop, one row buffer; nothing but the current row in flight per wavefront.
+#ifndef TTN_ADALN_BWD_ROW_BUFFERS
+#define TTN_ADALN_BWD_ROW_BUFFERS 1
+#endif
+#ifndef TTN_ADALN_BWD_PREFETCH_MID
+#define TTN_ADALN_BWD_PREFETCH_MID 0
+#endif
+#ifndef TTN_BWD_WAVES_PER_SIMD
+#define TTN_BWD_WAVES_PER_SIMD 1
+#endif
+
 namespace ttn {
 
 // Loads this sample's modulation row and returns t = rnd(1 + scale) packed in
@@ -130,15 +142,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // reductions reduce to sum_c gx and sum_c gx*x, both taken straight from packed
 // bf16 pairs, and dx becomes r*gx + x*K1 + K0 with per-row scalars K1, K0.
 template <typename T, int C, bool FROM_XNORM>
-__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 : 4) void adaln_bwd_kernel(
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void adaln_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
     const float *__restrict__ rstd, int64_t rows_per_sample, int blocks_per_sample) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
-    // fp32 rows of 3072 need 96 registers per row buffer: no room for a second one
-    constexpr bool kDoubleBuffer = !(sizeof(T) == 4 && C >= 1024);
+    // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
+    constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_ADALN_BWD_ROW_BUFFERS;
     __shared__ float lds[2 * C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
@@ -183,7 +195,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
         b.r = b.ok ? rstd[b.row] : 0.0f;
         b.mu = (!FROM_XNORM && b.ok) ? mean[b.row] : 0.0f;
     };
-    auto process = [&](const RowRegs &b) {
+    auto process = [&](const RowRegs &b, auto &&between_passes) {
         const float r = b.r, mu = b.mu;
         const float nmr = -(mu * r);  // xhat = x*r + nmr
         // pass 1: gx = rnd(g*t) kept packed; s1 = sum_c gx; s2 = sum_c gx * xhat
@@ -216,6 +228,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
         }
         s1 = group_sum<LANES>(s1);
         s2 = group_sum<LANES>(s2);
+        between_passes();
         if constexpr (kIsBf16<T> && !FROM_XNORM) s2 = r * (s2 - mu * s1);
         const float m1 = s1 / (float)C, m2 = s2 / (float)C;
         // dx = r*gx + xhat*k1 + k0,  k1 = -r*m2, k0 = -r*m1;  in terms of xin: r*gx + xin*K1 + K0
@@ -249,30 +262,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
     const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
     int64_t grp = (int64_t)slot * kRowWaves + wave;
-    if constexpr (kDoubleBuffer) {
-        if (grp < groups) {
-            RowRegs a, b;
-            fetch(a, grp);
-            for (;;) {
-                int64_t nxt = grp + stride;
-                bool more = nxt < groups;
-                if (more) fetch(b, nxt);
-                process(a);
-                if (!more) break;
-                grp = nxt + stride;
-                more = grp < groups;
-                if (more) fetch(a, grp);
-                process(b);
-                if (!more) break;
-            }
-        }
-    } else {
-        for (; grp < groups; grp += stride) {
-            RowRegs a;
-            fetch(a, grp);
-            process(a);
-        }
-    }
+    row_pipeline<kRowBuffers, TTN_ADALN_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
     flush_column_partials<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds);
 }
 
@@ -283,7 +273,7 @@ constexpr int kOneShotGrid = 1 << 20;
 #define TTN_ADALN_FWD_BLOCKS_PER_CU (C >= 1024 ? kOneShotGrid : 16)
 #endif
 #ifndef TTN_ADALN_BWD_BLOCKS_PER_CU
-#define TTN_ADALN_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 4)
+#define TTN_ADALN_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 3)
 #endif
 template <typename T, int C>
 struct AdalnTune {

@@ -186,6 +186,49 @@ __device__ __forceinline__ int wave_id_in_block() {
     return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }
 
+// Software pipeline over the rows of one wavefront.  `fetch(buf, grp)` issues the
+// loads of a row, `process(buf, mid)` consumes them and calls `mid()` once
+// between its two register passes.  grp advances by `stride` and is
+// wave-uniform, so every branch here is too.
+//   NBUF = 1 : plain loop (load, process, store; nothing else in flight).
+//   NBUF = 2, MID = false : the next row is requested before the current one is processed.
+//   NBUF = 2, MID = true  : the next row is requested half-way through the current one.
+template <int NBUF, bool MID, typename RowRegs, typename Fetch, typename Process>
+__device__ __forceinline__ void row_pipeline(int64_t grp, int64_t groups, int64_t stride, Fetch &&fetch,
+                                             Process &&process) {
+    static_assert(NBUF == 1 || NBUF == 2, "one or two row buffers");
+    auto nothing = [] {};
+    if constexpr (NBUF == 1) {
+        for (; grp < groups; grp += stride) {
+            RowRegs a;
+            fetch(a, grp);
+            process(a, nothing);
+        }
+    } else {
+        if (grp >= groups) return;
+        RowRegs buf[2];
+        fetch(buf[0], grp);
+        for (;;) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const int64_t ahead = grp + stride;
+                const bool more = ahead < groups;
+                auto request = [&] {
+                    if (more) fetch(buf[s ^ 1], ahead);
+                };
+                if constexpr (MID) {
+                    process(buf[s], request);
+                } else {
+                    request();
+                    process(buf[s], nothing);
+                }
+                if (!more) return;
+                grp = ahead;
+            }
+        }
+    }
+}
+
 // Adds this workgroup's per-lane column accumulators (acc[k][j] belongs to
 // column (k*LANES + l)*VEC + j) across the rows of each wavefront and across
 // wavefronts in fixed order, and writes one fp32 row of NSETS*C partial sums.

@@ -136,23 +136,25 @@ int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch
 }
 
 // ---- streaming copy ----------------------------------------------------------
-__global__ __launch_bounds__(256) void stream_copy_kernel(u32x4 *__restrict__ dst,
-                                                          const u32x4 *__restrict__ src, size_t n16) {
-    // six 16-byte accesses in flight per lane, the same depth as one 3072-wide bf16 row
+// The fastest plain copy found on this part, used as the yardstick next to the
+// kernels: one-shot grid, every wavefront copies one contiguous 6 KiB run (six
+// 16-byte accesses per lane, the shape of a 3072-wide bf16 row) and exits.
+__global__ __launch_bounds__(kRowThreads) void stream_copy_kernel(u32x4 *__restrict__ dst,
+                                                                  const u32x4 *__restrict__ src, size_t n16) {
     constexpr int kDepth = 6;
-    const size_t tile = (size_t)blockDim.x * kDepth;
-    for (size_t base = (size_t)blockIdx.x * tile; base < n16; base += (size_t)gridDim.x * tile) {
-        u32x4 v[kDepth];
+    const int lane = threadIdx.x & 63;
+    const size_t wave = (size_t)blockIdx.x * kRowWaves + wave_id_in_block();
+    const size_t base = wave * (kDepth * kWaveSize) + lane;
+    u32x4 v[kDepth];
 #pragma unroll
-        for (int k = 0; k < kDepth; ++k) {
-            const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
-            if (i < n16) v[k] = load16_stream(src + i);
-        }
+    for (int k = 0; k < kDepth; ++k) {
+        const size_t i = base + (size_t)k * kWaveSize;
+        if (i < n16) v[k] = load16_stream(src + i);
+    }
 #pragma unroll
-        for (int k = 0; k < kDepth; ++k) {
-            const size_t i = base + (size_t)k * blockDim.x + threadIdx.x;
-            if (i < n16) store16_stream(dst + i, v[k]);
-        }
+    for (int k = 0; k < kDepth; ++k) {
+        const size_t i = base + (size_t)k * kWaveSize;
+        if (i < n16) store16_stream(dst + i, v[k]);
     }
 }
 
@@ -188,14 +190,11 @@ int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) 
     if (bytes % 16) return fail(TT_NORM_EINVAL, "stream_copy: bytes (%zu) not a multiple of 16", bytes);
     if (!aligned16(dst) || !aligned16(src)) return fail(TT_NORM_EALIGN, "stream_copy: unaligned pointer");
     if (bytes == 0) return TT_NORM_OK;
-    int st = TT_NORM_OK;
-    const int cus = current_device_cus(&st);
-    if (st != TT_NORM_OK) return st;
     const size_t n16 = bytes / 16;
-    size_t blocks = (n16 + 256 * 6 - 1) / (256 * 6);
-    const size_t cap = (size_t)cus * 8;
-    if (blocks > cap) blocks = cap;
-    stream_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+    const size_t per_block = (size_t)kRowWaves * 6 * kWaveSize;
+    const size_t blocks = (n16 + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffULL) return fail(TT_NORM_EINVAL, "stream_copy: %zu bytes is too large for one launch", bytes);
+    stream_copy_kernel<<<dim3((unsigned)blocks), dim3(kRowThreads), 0, (hipStream_t)stream>>>(
         (u32x4 *)dst, (const u32x4 *)src, n16);
     return check_launch("stream copy launch");
 }

@@ -12,6 +12,18 @@
 #include "norm_device.h"
 #include "norm_host.h"
 
+// Backward pipeline shape at 3072 columns (measured back-to-back at 118 800 rows):
+// two row buffers with the next row requested half-way through the current one.
+#ifndef TTN_RMS_BWD_ROW_BUFFERS
+#define TTN_RMS_BWD_ROW_BUFFERS 2
+#endif
+#ifndef TTN_RMS_BWD_PREFETCH_MID
+#define TTN_RMS_BWD_PREFETCH_MID 1
+#endif
+#ifndef TTN_BWD_WAVES_PER_SIMD
+#define TTN_BWD_WAVES_PER_SIMD 1
+#endif
+
 namespace ttn {
 
 template <typename T, int C>
@@ -79,7 +91,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // keep about 48 KiB of reads in flight per compute unit, which is where this
 // memory system streams best; more resident wavefronts only add queueing.
 template <typename T, int C, bool FROM_OUT>
-__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 : 4) void rmsnorm_bwd_kernel(
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void rmsnorm_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ w, const float *__restrict__ rstd,
     int64_t rows) {
@@ -87,8 +99,8 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
     constexpr bool kPackedDot = kIsBf16<T> && !FROM_OUT;  // sum_c gy*x straight from bf16 pairs
-    // fp32 rows of 3072 need 96 registers per row buffer: no room for a second one
-    constexpr bool kDoubleBuffer = !(sizeof(T) == 4 && C >= 1024);
+    // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
+    constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_RMS_BWD_ROW_BUFFERS;
     __shared__ float lds[C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
@@ -130,7 +142,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
         }
         b.r = b.ok ? rstd[b.row] : 0.0f;
     };
-    auto process = [&](const RowRegs &b) {
+    auto process = [&](const RowRegs &b, auto &&between_passes) {
         const float r = b.r;
         // pass 1: gy = rnd(g*w), kept packed in the element type; row dot  sum_c gy * xs
         //   xs = x (native) or xhat = out / w (from the saved output)
@@ -155,6 +167,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
             }
         }
         dot = group_sum<LANES>(dot);
+        between_passes();
         // dx = gy*r + xs*coef
         const float coef = FROM_OUT ? -(r * (dot / (float)C)) : -((dot / (float)C) * r * r * r);
 
@@ -184,30 +197,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? 1 :
     const int64_t groups = (rows + RPW - 1) / RPW;
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave;
-    if constexpr (kDoubleBuffer) {
-        if (grp < groups) {
-            RowRegs a, b;
-            fetch(a, grp);
-            for (;;) {
-                int64_t nxt = grp + stride;
-                bool more = nxt < groups;
-                if (more) fetch(b, nxt);
-                process(a);
-                if (!more) break;
-                grp = nxt + stride;
-                more = grp < groups;
-                if (more) fetch(a, grp);
-                process(b);
-                if (!more) break;
-            }
-        }
-    } else {
-        for (; grp < groups; grp += stride) {
-            RowRegs a;
-            fetch(a, grp);
-            process(a);
-        }
-    }
+    row_pipeline<kRowBuffers, TTN_RMS_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
     flush_column_partials<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds);
 }
 
@@ -222,7 +212,7 @@ constexpr int kOneShot = 1 << 20;
 #define TTN_RMS_FWD_BLOCKS_PER_CU (C >= 1024 ? kOneShot : 16)
 #endif
 #ifndef TTN_RMS_BWD_BLOCKS_PER_CU
-#define TTN_RMS_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 4)
+#define TTN_RMS_BWD_BLOCKS_PER_CU (C >= 1024 ? 1 : 3)
 #endif
 template <typename T, int C>
 struct RmsTune {

@@ -330,3 +330,11 @@ def test_error_statuses(capi, gpu_device):
         capi.rmsnorm_forward(torch.zeros(4, 256, dtype=torch.bfloat16, device=gpu_device),
                              torch.ones(256, dtype=torch.bfloat16, device=gpu_device), EPS)
     torch.cuda.synchronize()
+
+
+def test_stream_copy_yardstick(capi, gpu_device):
+    for n in (16, 6144 * 4 * 3 + 16 * 5, 16 * 1000003):
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=gpu_device)
+        dst = torch.zeros_like(src)
+        capi.stream_copy(dst, src)
+        assert torch.equal(dst, src)
