@@ -95,6 +95,28 @@ int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, cons
                                  int64_t rows, int64_t cols, int dtype,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* Strided input: x is a 4-D view [n0, n1, n2, cols] whose last dimension is
+ * contiguous and whose other strides xs0..xs2 (in ELEMENTS, multiples of 16 bytes,
+ * >= 0) are arbitrary; out, dout and rstd are contiguous in logical order, i.e.
+ * row (i0*n1 + i1)*n2 + i2.  This is the per-head QK-norm call site: the reference
+ * normalises query.transpose(1, 2) (teletron/models/dit/dit_attention.py:201-212),
+ * a [B, H, S, D] view into the fused QKV projection, and first materialises a
+ * contiguous copy of it (teletron/models/dit/dit_fusedlayers.py:296); here the view
+ * is read in place.  dx is written through its own strides dxs0..dxs2, so the caller
+ * picks its layout.  Scratch: tt_rmsnorm_backward_workspace_bytes(n0*n1*n2, cols, dtype). */
+int tt_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void *weight,
+                               int64_t n0, int64_t n1, int64_t n2,
+                               int64_t xs0, int64_t xs1, int64_t xs2,
+                               int64_t cols, double eps, int dtype, void *stream);
+
+int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const void *x,
+                                const void *weight, const float *rstd,
+                                int64_t n0, int64_t n1, int64_t n2,
+                                int64_t xs0, int64_t xs1, int64_t xs2,
+                                int64_t dxs0, int64_t dxs1, int64_t dxs2,
+                                int64_t cols, int dtype,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
 /* -------------------------------------------------------------------- AdaLN
  * out = round(round(LN(x) * round(1 + scale[b])) + shift[b]),  LN without affine,
  * b = row / rows_per_sample  (teletron/models/dit/dit_fusedlayers.py:198,223).

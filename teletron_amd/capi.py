@@ -20,7 +20,7 @@ _DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
 EXPORTS = (
     "tt_norm_abi_version", "tt_norm_status_string", "tt_norm_last_error", "tt_norm_supported",
     "tt_rmsnorm_forward", "tt_rmsnorm_backward_workspace_bytes", "tt_rmsnorm_backward",
-    "tt_rmsnorm_backward_from_out",
+    "tt_rmsnorm_backward_from_out", "tt_rmsnorm_forward_strided", "tt_rmsnorm_backward_strided",
     "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
     "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
 )
@@ -52,6 +52,8 @@ def lib() -> ctypes.CDLL:
         L.tt_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64, ci]
         L.tt_rmsnorm_backward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp, sz, vp]
         L.tt_rmsnorm_backward_from_out.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp, sz, vp]
+        L.tt_rmsnorm_forward_strided.argtypes = [vp, vp, vp, vp] + [i64] * 7 + [dbl, ci, vp]
+        L.tt_rmsnorm_backward_strided.argtypes = [vp] * 6 + [i64] * 10 + [ci, vp, sz, vp]
         L.tt_adaln_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
         L.tt_adaln_forward_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
         L.tt_adaln_backward_workspace_bytes.restype = sz
@@ -120,6 +122,56 @@ def rmsnorm_backward(dout, x, weight, rstd, from_out: bool = False, dx=None, dwe
         fn = L.tt_rmsnorm_backward_from_out if from_out else L.tt_rmsnorm_backward
         _check(fn(_p(dx), _p(dweight), _p(dout), _p(x), _p(weight), _p(rstd), rows, cols, _dt(x),
                   _p(ws), n, _stream(x)), fn.__name__)
+    return dx, dweight
+
+
+def _view3(t: torch.Tensor):
+    """(sizes, strides) of t's leading dimensions padded to three; last dimension must be contiguous."""
+    if t.dim() < 1 or t.dim() > 4 or t.stride(-1) != 1:
+        raise ValueError("need a view of at most 4 dimensions with a contiguous last dimension")
+    sizes = [1] * (4 - t.dim()) + list(t.shape[:-1])
+    strides = [0] * (4 - t.dim()) + list(t.stride()[:-1])
+    return sizes, strides
+
+
+def dense_like_layout(x: torch.Tensor) -> torch.Tensor:
+    """An uninitialised tensor of x's shape whose memory order follows x's strides
+    (largest stride outermost) but without x's gaps."""
+    order = sorted(range(x.dim()), key=lambda d: (-x.stride(d), d))
+    buf = torch.empty([x.shape[d] for d in order], dtype=x.dtype, device=x.device)
+    inv = [order.index(d) for d in range(x.dim())]
+    return buf.permute(inv)
+
+
+def rmsnorm_forward_strided(x, weight, eps: float):
+    """x: any view (<= 4-D, contiguous last dim, 16-byte aligned strides); out is contiguous."""
+    if not x.is_cuda or not weight.is_cuda or not weight.is_contiguous():
+        raise ValueError("tensors must live on the GPU and weight must be contiguous")
+    cols = weight.numel()
+    (n0, n1, n2), (s0, s1, s2) = _view3(x)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    rstd = torch.empty(n0 * n1 * n2, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(lib().tt_rmsnorm_forward_strided(_p(out), _p(rstd), _p(x), _p(weight), n0, n1, n2, s0, s1, s2,
+                                                cols, eps, _dt(x), _stream(x)), "tt_rmsnorm_forward_strided")
+    return out, rstd
+
+
+def rmsnorm_backward_strided(dout, x, weight, rstd, dx=None):
+    """dout contiguous; x a view as in rmsnorm_forward_strided; dx (optional) any view of x's shape."""
+    _dense_gpu(dout, weight, rstd)
+    cols = weight.numel()
+    (n0, n1, n2), (s0, s1, s2) = _view3(x)
+    dx = dense_like_layout(x) if dx is None else dx
+    _, (d0, d1, d2) = _view3(dx)
+    dweight = torch.empty_like(weight)
+    with torch.cuda.device(x.device):
+        L = lib()
+        n = L.tt_rmsnorm_backward_workspace_bytes(n0 * n1 * n2, cols, _dt(x))
+        ws = _workspace(n, x)
+        _check(L.tt_rmsnorm_backward_strided(_p(dx), _p(dweight), _p(dout), _p(x), _p(weight), _p(rstd),
+                                             n0, n1, n2, s0, s1, s2, d0, d1, d2, cols, _dt(x), _p(ws), n,
+                                             _stream(x)), "tt_rmsnorm_backward_strided")
     return dx, dweight
 
 

@@ -72,12 +72,93 @@ void torch_launch_rms_backward_x(torch::Tensor &dinp, torch::Tensor &dweight, co
     rms_backward_impl(dinp, dweight, dout, input, weight, inv_variance, rows, cols, false);
 }
 
+// ---- strided views (no reference counterpart: the reference copies to contiguous first) ----
+struct View3 {
+    int64_t n[3], s[3];
+};
+
+// Leading dimensions of a <= 4-D view with contiguous last dimension, padded to three.
+static View3 view3(const torch::Tensor &t, int64_t cols, const char *name) {
+    TORCH_CHECK(t.dim() >= 1 && t.dim() <= 4, name, " must have 1 to 4 dimensions, got ", t.dim());
+    TORCH_CHECK(t.size(-1) == cols && t.stride(-1) == 1, name, " needs a contiguous last dimension of ", cols);
+    View3 v{{1, 1, 1}, {0, 0, 0}};
+    const int64_t lead = t.dim() - 1;
+    for (int64_t d = 0; d < lead; ++d) {
+        v.n[3 - lead + d] = t.size(d);
+        v.s[3 - lead + d] = t.stride(d);
+    }
+    return v;
+}
+
+// output (contiguous, input's shape) = rmsnorm(input view) * weight; inv_variance in output row order.
+void torch_launch_rms_forward_strided(torch::Tensor &output, const torch::Tensor &input,
+                                      const torch::Tensor &weight, double epsilon,
+                                      torch::Tensor &inv_variance) {
+    const auto dev = input.device();
+    TORCH_CHECK(input.is_cuda(), "input must be a GPU tensor");
+    check_dense_on(output, dev, "output");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(input, "input");
+    const int64_t cols = weight.numel();
+    const View3 v = view3(input, cols, "input");
+    const int64_t rows = v.n[0] * v.n[1] * v.n[2];
+    TORCH_CHECK(rows > 0, "input is empty");
+    check_elems(output, rows * cols, input.scalar_type(), "output");
+    check_elems(weight, cols, input.scalar_type(), "weight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_rmsnorm_forward_strided(output.data_ptr(), inv_variance.data_ptr<float>(), input.data_ptr(),
+                                        weight.data_ptr(), v.n[0], v.n[1], v.n[2], v.s[0], v.s[1], v.s[2], cols,
+                                        epsilon, dt, current_stream(input)),
+             "tt_rmsnorm_forward_strided");
+}
+
+// dinp: any view of input's shape (its strides choose the layout dx is written in); dout contiguous.
+void torch_launch_rms_backward_strided(torch::Tensor &dinp, torch::Tensor &dweight, const torch::Tensor &dout,
+                                       const torch::Tensor &input, const torch::Tensor &weight,
+                                       const torch::Tensor &inv_variance) {
+    const auto dev = dout.device();
+    TORCH_CHECK(input.is_cuda() && dinp.is_cuda(), "input and dinp must be GPU tensors");
+    TORCH_CHECK(input.device() == dev && dinp.device() == dev, "tensors are on different devices");
+    check_dense_on(dout, dev, "dout");
+    check_dense_on(dweight, dev, "dweight");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(dout, "dout");
+    const int64_t cols = weight.numel();
+    const View3 vx = view3(input, cols, "input");
+    const View3 vd = view3(dinp, cols, "dinp");
+    TORCH_CHECK(input.sizes() == dinp.sizes(), "dinp must have input's shape");
+    const int64_t rows = vx.n[0] * vx.n[1] * vx.n[2];
+    TORCH_CHECK(rows > 0, "input is empty");
+    TORCH_CHECK(input.scalar_type() == dout.scalar_type() && dinp.scalar_type() == dout.scalar_type(),
+                "input, dinp and dout must share a dtype");
+    check_elems(dout, rows * cols, dout.scalar_type(), "dout");
+    check_elems(weight, cols, dout.scalar_type(), "weight");
+    check_elems(dweight, cols, dout.scalar_type(), "dweight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_rmsnorm_backward_workspace_bytes(rows, cols, dt);
+    TORCH_CHECK(need > 0, "unsupported RMSNorm shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    raise_on(tt_rmsnorm_backward_strided(dinp.data_ptr(), dweight.data_ptr(), dout.data_ptr(), input.data_ptr(),
+                                         weight.data_ptr(), inv_variance.data_ptr<float>(), vx.n[0], vx.n[1],
+                                         vx.n[2], vx.s[0], vx.s[1], vx.s[2], vd.s[0], vd.s[1], vd.s[2], cols, dt,
+                                         ws.data_ptr(), need, current_stream(dout)),
+             "tt_rmsnorm_backward_strided");
+}
+
 PYBIND11_MODULE(fused_rmsnorm, m) {
     m.def("torch_launch_rms_forward", &torch_launch_rms_forward, "RMSNorm forward kernel");
     m.def("torch_launch_rms_backward", &torch_launch_rms_backward,
           "RMSNorm backward kernel (from the saved forward output)");
     m.def("torch_launch_rms_backward_x", &torch_launch_rms_backward_x,
           "RMSNorm backward kernel (from the saved input)");
+    m.def("torch_launch_rms_forward_strided", &torch_launch_rms_forward_strided,
+          "RMSNorm forward kernel reading a strided view (contiguous last dimension) in place");
+    m.def("torch_launch_rms_backward_strided", &torch_launch_rms_backward_strided,
+          "RMSNorm backward kernel for a strided input view; dx is written through dinp's strides");
     m.def("supported", [](int64_t cols, const torch::Tensor &like) {
         return tt_norm_supported(cols, like.scalar_type() == at::kBFloat16 ? TT_NORM_BF16
                                        : like.scalar_type() == at::kFloat  ? TT_NORM_F32 : -1) != 0;

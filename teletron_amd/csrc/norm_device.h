@@ -206,25 +206,27 @@ __device__ __forceinline__ void row_pipeline(int64_t grp, int64_t groups, int64_
         }
     } else {
         if (grp >= groups) return;
-        RowRegs buf[2];
-        fetch(buf[0], grp);
-        for (;;) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const int64_t ahead = grp + stride;
-                const bool more = ahead < groups;
-                auto request = [&] {
-                    if (more) fetch(buf[s ^ 1], ahead);
-                };
-                if constexpr (MID) {
-                    process(buf[s], request);
-                } else {
-                    request();
-                    process(buf[s], nothing);
-                }
-                if (!more) return;
-                grp = ahead;
+        RowRegs buf0, buf1;
+        fetch(buf0, grp);
+        // one row: process `cur`, requesting the row after it into `nxt`; false when it was the last
+        auto step = [&](RowRegs &cur, RowRegs &nxt) -> bool {
+            const int64_t ahead = grp + stride;
+            const bool more = ahead < groups;
+            auto request = [&] {
+                if (more) fetch(nxt, ahead);
+            };
+            if constexpr (MID) {
+                process(cur, request);
+            } else {
+                request();
+                process(cur, nothing);
             }
+            grp = ahead;
+            return more;
+        };
+        for (;;) {
+            if (!step(buf0, buf1)) return;
+            if (!step(buf1, buf0)) return;
         }
     }
 }

@@ -26,10 +26,67 @@
 
 namespace ttn {
 
-template <typename T, int C>
+// ---- where a wavefront's rows live ---------------------------------------------
+// A row map turns (wavefront group index, row within the wavefront) into the
+// row's logical number -- its index in the contiguous tensors (out, dout) and in
+// the per-row statistics -- and its element offsets in the tensors that may be
+// strided (x and, for backward, dx).
+struct RowAddr {
+    int64_t row;   // logical row number
+    int64_t xoff;  // element offset of the row in x
+    int64_t doff;  // element offset of the row in dx (backward only)
+    bool ok;
+};
+
+// Row-major contiguous [rows, C].
+struct DenseRows {
+    int64_t rows;
+    template <int RPW>
+    __device__ __forceinline__ int64_t groups() const { return (rows + RPW - 1) / RPW; }
+    template <int RPW, int C>
+    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub) const {
+        RowAddr a;
+        a.row = grp * RPW + sub;
+        a.ok = a.row < rows;
+        a.xoff = a.doff = a.row * C;
+        return a;
+    }
+};
+
+// A 4-D view [n0, n1, n2, C] with contiguous last dimension and arbitrary other
+// strides (in elements); logical row number (i0*n1 + i1)*n2 + i2.  This is the
+// per-head QK-norm input: query.transpose(1, 2) is [B, H, S, D] with strides
+// (S*H*3D, 3D, H*3D, 1) inside the fused QKV projection output.
+// Traversal: a wavefront takes RPW consecutive i2 of one (i0, i1) -- so what it
+// writes to the contiguous side is one unbroken run -- and consecutive wavefronts
+// take consecutive i1 for the same i2 tile, so the workgroups running at the
+// same time read neighbouring pieces of the strided side.
+struct Strided3Rows {
+    int64_t n0, n1, n2;
+    int64_t xs0, xs1, xs2;
+    int64_t ds0, ds1, ds2;
+    template <int RPW>
+    __device__ __forceinline__ int64_t groups() const { return n0 * n1 * ((n2 + RPW - 1) / RPW); }
+    template <int RPW, int C>
+    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub) const {
+        const int64_t tiles2 = (n2 + RPW - 1) / RPW;
+        const int64_t i1 = grp % n1;
+        const int64_t q = grp / n1;
+        const int64_t i2 = (q % tiles2) * RPW + sub;
+        const int64_t i0 = q / tiles2;
+        RowAddr a;
+        a.ok = i2 < n2;
+        a.row = (i0 * n1 + i1) * n2 + i2;
+        a.xoff = i0 * xs0 + i1 * xs1 + i2 * xs2;
+        a.doff = i0 * ds0 + i1 * ds1 + i2 * ds2;
+        return a;
+    }
+};
+
+template <typename T, int C, typename Map>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void rmsnorm_fwd_kernel(
     T *__restrict__ out, float *__restrict__ rstd, const T *__restrict__ x,
-    const T *__restrict__ w, int64_t rows, float eps) {
+    const T *__restrict__ w, const Map map, float eps) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
@@ -42,13 +99,14 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) wr[k] = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
 
-    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t groups = map.template groups<RPW>();
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
         keep_packed(wr);
-        const int64_t row = grp * RPW + sub;
-        const bool ok = row < rows;
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(x + row * C) + l;
+        const RowAddr at = map.template locate<RPW, C>(grp, sub);
+        const int64_t row = at.row;
+        const bool ok = at.ok;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(x + at.xoff) + l;
         u32x4 xr[CHUNKS];
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
@@ -90,11 +148,11 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // processed (two row buffers, ping-pong).  Few, fat, always-loading wavefronts
 // keep about 48 KiB of reads in flight per compute unit, which is where this
 // memory system streams best; more resident wavefronts only add queueing.
-template <typename T, int C, bool FROM_OUT>
+template <typename T, int C, bool FROM_OUT, typename Map>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void rmsnorm_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ w, const float *__restrict__ rstd,
-    int64_t rows) {
+    const Map map) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
@@ -127,20 +185,21 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     struct RowRegs {
         u32x4 g[CHUNKS], x[CHUNKS];
         float r;
-        int64_t row;
+        int64_t doff;
         bool ok;
     };
     auto fetch = [&](RowRegs &b, int64_t grp) {
-        b.row = grp * RPW + sub;
-        b.ok = b.row < rows;
-        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
+        const RowAddr at = map.template locate<RPW, C>(grp, sub);
+        b.ok = at.ok;
+        b.doff = at.doff;
+        const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
-        b.r = b.ok ? rstd[b.row] : 0.0f;
+        b.r = b.ok ? rstd[at.row] : 0.0f;
     };
     auto process = [&](const RowRegs &b, auto &&between_passes) {
         const float r = b.r;
@@ -171,7 +230,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         // dx = gy*r + xs*coef
         const float coef = FROM_OUT ? -(r * (dot / (float)C)) : -((dot / (float)C) * r * r * r);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.row * C) + l;
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.doff) + l;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
@@ -194,7 +253,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         }
     };
 
-    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t groups = map.template groups<RPW>();
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave;
     row_pipeline<kRowBuffers, TTN_RMS_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
@@ -220,27 +279,30 @@ struct RmsTune {
     static constexpr int kBwdBlocksPerCu = TTN_RMS_BWD_BLOCKS_PER_CU;
 };
 
-template <typename T, int C>
-static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *w, int64_t rows,
-                             double eps, hipStream_t stream) {
+template <typename T, int C, typename Map>
+static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *w, const Map &map,
+                             int64_t rows, double eps, hipStream_t stream) {
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
     const RowPlan p = make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kFwdBlocksPerCu, cus);
-    rmsnorm_fwd_kernel<T, C><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-        (T *)out, rstd, (const T *)x, (const T *)w, rows, (float)eps);
+    if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "rmsnorm forward: grid too large");
+    rmsnorm_fwd_kernel<T, C, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+        (T *)out, rstd, (const T *)x, (const T *)w, map, (float)eps);
     return check_launch("rmsnorm forward launch");
 }
 
+// The backward grid (and with it the scratch size) depends on the row count only,
+// also for strided views: a persistent grid covers any traversal.
 template <typename T, int C>
 static RowPlan rmsnorm_backward_plan(int64_t rows, int cus) {
     return make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kBwdBlocksPerCu, cus);
 }
 
-template <typename T, int C, bool FROM_OUT>
+template <typename T, int C, bool FROM_OUT, typename Map>
 static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin, const void *w,
-                              const float *rstd, int64_t rows, int dtype, void *ws, size_t ws_bytes,
-                              hipStream_t stream) {
+                              const float *rstd, const Map &map, int64_t rows, int dtype, void *ws,
+                              size_t ws_bytes, hipStream_t stream) {
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -248,8 +310,8 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
     const size_t need = (size_t)p.blocks * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
-    rmsnorm_bwd_kernel<T, C, FROM_OUT><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, rows);
+    rmsnorm_bwd_kernel<T, C, FROM_OUT, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, map);
     st = check_launch("rmsnorm backward launch");
     if (st != TT_NORM_OK) return st;
     return launch_colreduce(dw, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);
@@ -290,7 +352,7 @@ int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight
     int st = check_rms_args("tt_rmsnorm_forward", rows, cols, dtype, {out, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward: null rstd");
-#define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, rows, eps, (hipStream_t)stream)
+#define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, DenseRows{rows}, rows, eps, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
 }
@@ -312,8 +374,8 @@ int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x
     if (st != TT_NORM_OK) return st;
     if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
 #define CALL(T, C)                                                                                  \
-    return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, rows, dtype, workspace, \
-                                           workspace_bytes, (hipStream_t)stream)
+    return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, DenseRows{rows}, rows, dtype, \
+                                           workspace, workspace_bytes, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
 }
@@ -325,8 +387,58 @@ int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, cons
     if (st != TT_NORM_OK) return st;
     if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_from_out: null dweight/rstd");
 #define CALL(T, C)                                                                                   \
-    return rmsnorm_backward_t<T, C, true>(dx, dweight, dout, out, weight, rstd, rows, dtype, workspace, \
-                                          workspace_bytes, (hipStream_t)stream)
+    return rmsnorm_backward_t<T, C, true>(dx, dweight, dout, out, weight, rstd, DenseRows{rows}, rows, dtype, \
+                                          workspace, workspace_bytes, (hipStream_t)stream)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+static int check_strided(const char *who, int64_t n0, int64_t n1, int64_t n2, int64_t cols, int dtype,
+                         const int64_t (&strides)[3], const char *what) {
+    if (n0 <= 0 || n1 <= 0 || n2 <= 0)
+        return fail(TT_NORM_EINVAL, "%s: sizes [%lld, %lld, %lld]", who, (long long)n0, (long long)n1, (long long)n2);
+    if (!tt_norm_supported(cols, dtype)) return TT_NORM_OK;  // reported by the common check
+    const int64_t vec = dtype == TT_NORM_BF16 ? 8 : 4;
+    for (int64_t s : strides)
+        if (s < 0 || s % vec != 0)
+            return fail(TT_NORM_EALIGN, "%s: %s stride %lld is not a non-negative multiple of %lld elements (16 bytes)",
+                        who, what, (long long)s, (long long)vec);
+    return TT_NORM_OK;
+}
+
+int tt_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void *weight, int64_t n0,
+                               int64_t n1, int64_t n2, int64_t xs0, int64_t xs1, int64_t xs2, int64_t cols,
+                               double eps, int dtype, void *stream) {
+    const int64_t xs[3] = {xs0, xs1, xs2};
+    int st = check_strided("tt_rmsnorm_forward_strided", n0, n1, n2, cols, dtype, xs, "x");
+    if (st != TT_NORM_OK) return st;
+    const int64_t rows = n0 * n1 * n2;
+    st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight});
+    if (st != TT_NORM_OK) return st;
+    if (!rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward_strided: null rstd");
+    const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, 0, 0, 0};
+#define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, map, rows, eps, (hipStream_t)stream)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const void *x, const void *weight,
+                                const float *rstd, int64_t n0, int64_t n1, int64_t n2, int64_t xs0,
+                                int64_t xs1, int64_t xs2, int64_t dxs0, int64_t dxs1, int64_t dxs2,
+                                int64_t cols, int dtype, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+    const int64_t xs[3] = {xs0, xs1, xs2}, ds[3] = {dxs0, dxs1, dxs2};
+    int st = check_strided("tt_rmsnorm_backward_strided", n0, n1, n2, cols, dtype, xs, "x");
+    if (st == TT_NORM_OK) st = check_strided("tt_rmsnorm_backward_strided", n0, n1, n2, cols, dtype, ds, "dx");
+    if (st != TT_NORM_OK) return st;
+    const int64_t rows = n0 * n1 * n2;
+    st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight});
+    if (st != TT_NORM_OK) return st;
+    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_strided: null dweight/rstd");
+    const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, dxs0, dxs1, dxs2};
+#define CALL(T, C)                                                                                       \
+    return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, map, rows, dtype, workspace, \
+                                           workspace_bytes, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
 }

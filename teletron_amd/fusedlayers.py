@@ -251,31 +251,55 @@ class FusedAdaLayerNormZeroSingle(_AdaLNZeroBase):
         return self._modulate(x, scale_msa, shift_msa), gate_msa
 
 
+def _strided_rows_ok(x: torch.Tensor) -> bool:
+    """True if x can be normalised in place as a strided view: at most 4-D, last
+    dimension contiguous, every other stride a non-negative multiple of 16 bytes."""
+    if x.is_contiguous() or x.dim() > 4 or x.dim() < 2 or x.stride(-1) != 1:
+        return False
+    vec = 16 // x.element_size()
+    return all(st >= 0 and st % vec == 0 for st in x.stride()[:-1]) and x.data_ptr() % 16 == 0
+
+
+def _dense_like_layout(x: torch.Tensor) -> torch.Tensor:
+    """Uninitialised tensor of x's shape laid out in x's dimension order but without its gaps."""
+    order = sorted(range(x.dim()), key=lambda d: (-x.stride(d), d))
+    buf = torch.empty([x.shape[d] for d in order], dtype=x.dtype, device=x.device)
+    return buf.permute([order.index(d) for d in range(x.dim())])
+
+
 class RMSNormModelFunction(Function):
     """out = (x * rsqrt(mean(x^2) + eps)) * weight over the last `cols` elements.
 
     apply(x, weight, epsilon, cols) -> out, with gradients for x and weight
-    (dit_fusedlayers.py:281,317)."""
+    (dit_fusedlayers.py:281,317).  A non-contiguous view with a contiguous last
+    dimension -- the attention caller passes query.transpose(1, 2),
+    dit_attention.py:201-212 -- is read in place; the reference copies it first
+    (dit_fusedlayers.py:296).  The output is contiguous either way."""
 
     @staticmethod
     def forward(ctx, x, weight, epsilon, cols):
         ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
         _require_gpu(x, "RMSNormModelFunction")
-        x = x.contiguous()
         if cols not in SUPPORTED_COLS or x.numel() == 0 or x.numel() % cols != 0:
             raise ValueError(f"Input size {x.numel()} not divisible by cols {cols} or unsupported cols value "
                              f"(supported: {SUPPORTED_COLS})")
         if weight.numel() != cols:
             raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
+        strided = x.shape[-1] == cols and _strided_rows_ok(x)
+        if not strided:
+            x = x.contiguous()
         w = weight.contiguous()
         if w.dtype != x.dtype:
             w = w.to(x.dtype)
         rows = x.numel() // cols
-        out = torch.empty_like(x)
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         invvar = torch.empty(rows, device=x.device, dtype=torch.float32)
-        ext.torch_launch_rms_forward(out, x, w, rows, cols, float(epsilon), invvar)
+        if strided:
+            ext.torch_launch_rms_forward_strided(out, x, w, float(epsilon), invvar)
+        else:
+            ext.torch_launch_rms_forward(out, x, w, rows, cols, float(epsilon), invvar)
         ctx.save_for_backward(x, w, invvar)
-        ctx.rows, ctx.cols = rows, cols
+        ctx.rows, ctx.cols, ctx.strided = rows, cols, strided
         ctx.w_shape, ctx.w_dtype = weight.shape, weight.dtype
         return out
 
@@ -285,10 +309,14 @@ class RMSNormModelFunction(Function):
         grad_output = grad_output.contiguous()
         if grad_output.dtype != x.dtype:
             grad_output = grad_output.to(x.dtype)
-        grad_input = torch.empty_like(x)
         grad_weight = torch.empty_like(w)
-        fused_rmsnorm.torch_launch_rms_backward_x(grad_input, grad_weight, grad_output, x, w, invvar,
-                                                  ctx.rows, ctx.cols)
+        if ctx.strided:
+            grad_input = _dense_like_layout(x)   # x's dimension order, so the transposed view's grad is cheap to undo
+            fused_rmsnorm.torch_launch_rms_backward_strided(grad_input, grad_weight, grad_output, x, w, invvar)
+        else:
+            grad_input = torch.empty_like(x)
+            fused_rmsnorm.torch_launch_rms_backward_x(grad_input, grad_weight, grad_output, x, w, invvar,
+                                                      ctx.rows, ctx.cols)
         return grad_input, grad_weight.reshape(ctx.w_shape).to(ctx.w_dtype), None, None
 
 

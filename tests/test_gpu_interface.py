@@ -195,3 +195,46 @@ def test_reference_signature_extension_calls(FL, gpu_device):
     assert torch.equal(out2, output)
     with pytest.raises(RuntimeError, match="elements"):
         FL.fused_rmsnorm.torch_launch_rms_forward(output, x, w, rows + 1, 128, EPS, invvar)
+
+
+def test_rmsnorm_function_reads_qkv_view_in_place(FL, gpu_device):
+    """q and k sliced out of a fused QKV projection and transposed, as in the attention module:
+    the function must not need a contiguous copy, and gradients must flow back into the projection."""
+    B, S, H, D = 1, 513, 24, 128
+    gen = torch.Generator().manual_seed(50)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()
+    w = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    gq = torch.randn(B, H, S, D, generator=gen).bfloat16()
+    gk = torch.randn(B, H, S, D, generator=gen).bfloat16()
+
+    def run(mixed_t, w_t, norm):
+        mixed_t = mixed_t.clone().requires_grad_(True)
+        w_t = w_t.clone().requires_grad_(True)
+        q, k, v = torch.split(mixed_t, [D, D, D], dim=3)
+        qn = norm(q.transpose(1, 2), w_t)
+        kn = norm(k.transpose(1, 2), w_t)
+        (qn * gq.to(qn.device)).sum().backward(retain_graph=True)
+        (kn * gk.to(kn.device)).sum().backward()
+        return qn.detach(), kn.detach(), mixed_t.grad, w_t.grad
+
+    want = run(mixed, w, lambda x, wt: O.eager_rmsnorm(x, wt, EPS))
+    calls = {"strided": 0}
+    orig = FL.fused_rmsnorm.torch_launch_rms_forward_strided
+
+    def counting(*a):
+        calls["strided"] += 1
+        return orig(*a)
+
+    FL.fused_rmsnorm.torch_launch_rms_forward_strided = counting
+    try:
+        got = run(mixed.to(gpu_device), w.to(gpu_device),
+                  lambda x, wt: FL.RMSNormModelFunction.apply(x, wt, EPS, D))
+    finally:
+        FL.fused_rmsnorm.torch_launch_rms_forward_strided = orig
+    assert calls["strided"] == 2                       # both q and k took the in-place path
+    fwd_ok(got[0], want[0], O.rmsnorm_excuse(want[0]))
+    fwd_ok(got[1], want[1], O.rmsnorm_excuse(want[1]))
+    assert O.frac_outside(got[2].cpu(), want[2], 1e-2, 1e-3) == 0.0      # d(mixed): q and k slots filled, v zero
+    assert got[2][..., 2 * D:].abs().max() == 0
+    # dweight sums two accumulated calls in bf16 on both sides: allow one extra bf16 rounding
+    assert O.frac_outside(got[3].cpu(), want[3], 2e-2, 1e-3) == 0.0

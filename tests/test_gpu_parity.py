@@ -338,3 +338,70 @@ def test_stream_copy_yardstick(capi, gpu_device):
         dst = torch.zeros_like(src)
         capi.stream_copy(dst, src)
         assert torch.equal(dst, src)
+
+
+# ------------------------------------------- strided views (QK-norm call site)
+
+def _qkv_views(B, S, H, D, dtype, seed, device):
+    """query/key as the attention caller sees them: slices of a fused [B, S, H, 3D] projection,
+    transposed to [B, H, S, D] (dit_attention.py:149-203)."""
+    gen = torch.Generator().manual_seed(seed)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).to(dtype)
+    q_cpu, k_cpu, _ = torch.split(mixed, [D, D, D], dim=3)
+    mixed_g = mixed.to(device)
+    q_g, k_g, _ = torch.split(mixed_g, [D, D, D], dim=3)
+    return q_cpu.transpose(1, 2), k_cpu.transpose(1, 2), q_g.transpose(1, 2), k_g.transpose(1, 2)
+
+
+@pytest.mark.parametrize("B,S,H", [(1, 1001, 24), (2, 37, 6), (1, 3, 1)])
+def test_rmsnorm_strided_qk_view_matches_eager(capi, gpu_device, B, S, H):
+    D = 128
+    q_cpu, k_cpu, q_g, k_g = _qkv_views(B, S, H, D, torch.bfloat16, 5, gpu_device)
+    gen = torch.Generator().manual_seed(6)
+    w = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    grad = torch.randn(B, H, S, D, generator=gen).bfloat16()
+    for x_cpu, x_g in ((q_cpu, q_g), (k_cpu, k_g)):
+        assert not x_g.is_contiguous()
+        want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(x_cpu, w, grad)
+        out, rstd = capi.rmsnorm_forward_strided(x_g, w.to(gpu_device), EPS)
+        assert out.is_contiguous() and out.shape == (B, H, S, D)
+        assert_fwd_bf16(out, want_out, None, "out")
+        # identical to the dense kernel on a materialised copy (same per-row arithmetic)
+        out_dense, rstd_dense = capi.rmsnorm_forward(x_g.contiguous(), w.to(gpu_device), EPS)
+        assert torch.equal(out, out_dense) and torch.equal(rstd, rstd_dense)
+        dx, dw = capi.rmsnorm_backward_strided(grad.to(gpu_device), x_g, w.to(gpu_device), rstd)
+        assert dx.shape == x_g.shape and dx.transpose(1, 2).is_contiguous()   # laid out in x's dimension order
+        assert_grad_bf16(dx, want_dx, "dx")
+        assert_grad_bf16(dw, want_dw, "dweight")
+        dx_dense, _ = capi.rmsnorm_backward(grad.to(gpu_device), x_g.contiguous(), w.to(gpu_device), rstd_dense)
+        assert torch.equal(dx.contiguous(), dx_dense)
+
+
+def test_rmsnorm_strided_3072_transposed_and_fp32(capi, gpu_device):
+    """[S, B, C] activations viewed as [B, S, C] (the blocks transpose between the two layouts)."""
+    S, B, C = 301, 2, 3072
+    for dtype in (torch.bfloat16, torch.float32):
+        d = O.make_rmsnorm_inputs((S, B), C, dtype, seed=9)
+        xv_cpu = d["x"].transpose(0, 1)
+        gv = d["grad"].transpose(0, 1).contiguous()
+        want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(xv_cpu, d["weight"], gv)
+        x_g = d["x"].to(gpu_device).transpose(0, 1)
+        w_g = d["weight"].to(gpu_device)
+        out, rstd = capi.rmsnorm_forward_strided(x_g, w_g, EPS)
+        dx, dw = capi.rmsnorm_backward_strided(gv.to(gpu_device), x_g, w_g, rstd)
+        if dtype == torch.bfloat16:
+            assert_fwd_bf16(out, want_out, None, "out")
+            assert_grad_bf16(dx, want_dx, "dx")
+            assert_grad_bf16(dw, want_dw, "dweight")
+        else:
+            torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(dx.cpu(), want_dx, rtol=1e-4, atol=1e-5)
+
+
+def test_rmsnorm_strided_rejects_unaligned_strides(capi, gpu_device):
+    base = torch.zeros(4, 10, 132, dtype=torch.bfloat16, device=gpu_device)
+    view = base[:, :, :128]                      # row stride 132 elements = 264 bytes: not 16-byte aligned
+    w = torch.ones(128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(capi.NormError) as e:
+        capi.rmsnorm_forward_strided(view, w, EPS)
+    assert e.value.status == 3
