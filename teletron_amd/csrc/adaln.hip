@@ -25,6 +25,13 @@
 #ifndef TTN_ADALN_BWD_PREFETCH_MID
 #define TTN_ADALN_BWD_PREFETCH_MID 0
 #endif
+// Dynamic LDS requested by the forward launch (0: none).  Only a throttle on how many
+// one-shot workgroups a compute unit holds at once; the kernel does not touch it.
+// AdaLN forward spends longer in the ALU per row than RMSNorm forward and wants all the
+// wavefronts its registers allow (16 per compute unit), so no throttle here.
+#ifndef TTN_ADALN_FWD_DYN_LDS
+#define TTN_ADALN_FWD_DYN_LDS 0
+#endif
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
@@ -296,7 +303,7 @@ static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, con
     const RowPlan p = make_row_plan(a.batch, a.rows_per_sample, RowGeom<T, C>::RPW,
                                     AdalnTune<T, C>::kFwdBlocksPerCu, cus);
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln forward: grid too large");
-    adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+    adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
         (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
         a.rows_per_sample, p.blocks_per_sample, (float)a.eps);
     return check_launch("adaln forward launch");
