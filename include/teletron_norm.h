@@ -157,6 +157,16 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                  void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------- measurement
+ * Arms a pair of HIP events (hipEvent_t passed as void*, created by the caller with
+ * timing enabled) for the NEXT row kernel launched from this thread: `start` is
+ * recorded on that launch's stream immediately before the row kernel and `stop`
+ * immediately after it, i.e. before the column reducer of a backward call.  One shot:
+ * the pair is disarmed once used.  No counterpart in the reference (which has no
+ * instrumentation); it exists so that a benchmark can time exactly the kernel a
+ * profiler reports.  Pass NULLs to disarm. */
+int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event);
+
+/*
  * Plain streaming copy of `bytes` (multiple of 16) from src to dst with the
  * same 128-bit access pattern as the kernels: the achievable-bandwidth
  * yardstick the benchmark prints next to each result. */

@@ -23,6 +23,7 @@ EXPORTS = (
     "tt_rmsnorm_backward_from_out", "tt_rmsnorm_forward_strided", "tt_rmsnorm_backward_strided",
     "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
     "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
+    "tt_norm_profile_next_row_kernel",
 )
 
 
@@ -61,6 +62,7 @@ def lib() -> ctypes.CDLL:
         L.tt_adaln_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_from_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
+        L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
     return _lib
 

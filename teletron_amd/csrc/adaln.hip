@@ -303,9 +303,12 @@ static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, con
     const RowPlan p = make_row_plan(a.batch, a.rows_per_sample, RowGeom<T, C>::RPW,
                                     AdalnTune<T, C>::kFwdBlocksPerCu, cus);
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln forward: grid too large");
-    adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
-        (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
-        a.rows_per_sample, p.blocks_per_sample, (float)a.eps);
+    {
+        RowKernelProfile prof(a.stream);
+        adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
+            (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
+            a.rows_per_sample, p.blocks_per_sample, (float)a.eps);
+    }
     return check_launch("adaln forward launch");
 }
 
@@ -326,9 +329,12 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
     const size_t need = (size_t)p.blocks * 2 * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
-    adaln_bwd_kernel<T, C, FROM_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
-        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
-        a.rows_per_sample, p.blocks_per_sample);
+    {
+        RowKernelProfile prof(a.stream);
+        adaln_bwd_kernel<T, C, FROM_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+            (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
+            a.rows_per_sample, p.blocks_per_sample);
+    }
     st = check_launch("adaln backward launch");
     if (st != TT_NORM_OK) return st;
     return launch_colreduce(dscale, dshift, (const float *)ws, a.batch, p.blocks_per_sample, C, 2 * C,

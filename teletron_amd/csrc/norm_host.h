@@ -25,6 +25,20 @@ inline size_t elem_bytes(int dtype) { return dtype == TT_NORM_BF16 ? 2 : 4; }
 // Checks the last launch on this thread; returns TT_NORM_OK or TT_NORM_EHIP.
 int check_launch(const char *what);
 
+// Brackets the row-kernel launch made inside its scope with the event pair armed by
+// tt_norm_profile_next_row_kernel (if any), on `stream`; disarms the pair.
+class RowKernelProfile {
+public:
+    explicit RowKernelProfile(hipStream_t stream);
+    ~RowKernelProfile();
+    RowKernelProfile(const RowKernelProfile &) = delete;
+    RowKernelProfile &operator=(const RowKernelProfile &) = delete;
+
+private:
+    hipStream_t stream_;
+    hipEvent_t stop_;
+};
+
 // ---- launch geometry -------------------------------------------------------
 // Every row kernel runs as a persistent 1-D grid of `batch * blocks_per_sample`
 // workgroups of kRowWaves wavefronts.  Workgroup i serves sample

@@ -44,6 +44,19 @@ int current_device_cus(int *status) {
     return cus;
 }
 
+static thread_local hipEvent_t g_profile_start = nullptr;
+static thread_local hipEvent_t g_profile_stop = nullptr;
+
+RowKernelProfile::RowKernelProfile(hipStream_t stream) : stream_(stream), stop_(g_profile_stop) {
+    if (g_profile_start) (void)hipEventRecord(g_profile_start, stream_);
+    g_profile_start = nullptr;
+    g_profile_stop = nullptr;
+}
+
+RowKernelProfile::~RowKernelProfile() {
+    if (stop_) (void)hipEventRecord(stop_, stream_);
+}
+
 int check_launch(const char *what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(TT_NORM_EHIP, "%s: %s", what, hipGetErrorString(e));
@@ -183,6 +196,14 @@ const char *tt_norm_last_error(void) { return g_last_error; }
 int tt_norm_supported(int64_t cols, int dtype) {
     if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F32) return 0;
     return (cols == 128 || cols == 3072) ? 1 : 0;
+}
+
+int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event) {
+    if ((start_event == nullptr) != (stop_event == nullptr))
+        return fail(TT_NORM_EINVAL, "profile_next_row_kernel: pass both events or neither");
+    g_profile_start = (hipEvent_t)start_event;
+    g_profile_stop = (hipEvent_t)stop_event;
+    return TT_NORM_OK;
 }
 
 int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {

@@ -294,8 +294,11 @@ static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *
     if (st != TT_NORM_OK) return st;
     const RowPlan p = make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kFwdBlocksPerCu, cus);
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "rmsnorm forward: grid too large");
-    rmsnorm_fwd_kernel<T, C, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_RMS_FWD_DYN_LDS, stream>>>(
-        (T *)out, rstd, (const T *)x, (const T *)w, map, (float)eps);
+    {
+        RowKernelProfile prof(stream);
+        rmsnorm_fwd_kernel<T, C, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_RMS_FWD_DYN_LDS, stream>>>(
+            (T *)out, rstd, (const T *)x, (const T *)w, map, (float)eps);
+    }
     return check_launch("rmsnorm forward launch");
 }
 
@@ -317,8 +320,11 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
     const size_t need = (size_t)p.blocks * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
-    rmsnorm_bwd_kernel<T, C, FROM_OUT, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-        (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, map);
+    {
+        RowKernelProfile prof(stream);
+        rmsnorm_bwd_kernel<T, C, FROM_OUT, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+            (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, map);
+    }
     st = check_launch("rmsnorm backward launch");
     if (st != TT_NORM_OK) return st;
     return launch_colreduce(dw, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);

@@ -405,3 +405,28 @@ def test_rmsnorm_strided_rejects_unaligned_strides(capi, gpu_device):
     with pytest.raises(capi.NormError) as e:
         capi.rmsnorm_forward_strided(view, w, EPS)
     assert e.value.status == 3
+
+
+def test_profile_hook_brackets_the_row_kernel(capi, gpu_device):
+    """tt_norm_profile_next_row_kernel: one shot, records on the launch stream around the row kernel."""
+    hip = ctypes.CDLL("libamdhip64.so")
+    ev = [ctypes.c_void_p() for _ in range(2)]
+    for e in ev:
+        assert hip.hipEventCreate(ctypes.byref(e)) == 0
+    L = capi.lib()
+    assert L.tt_norm_profile_next_row_kernel(ev[0], None) == 1          # both or neither
+    d = dev(O.make_rmsnorm_inputs((20000,), 3072, torch.bfloat16, seed=2), gpu_device)
+    out, rstd = capi.rmsnorm_forward(d["x"], d["weight"], EPS)
+    assert L.tt_norm_profile_next_row_kernel(ev[0], ev[1]) == 0
+    dx, dw = capi.rmsnorm_backward(d["grad"], d["x"], d["weight"], rstd)
+    torch.cuda.synchronize()
+    ms = ctypes.c_float()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), ev[0], ev[1]) == 0
+    assert 0.01 < ms.value < 5.0                                         # 20 000 rows: tens of microseconds
+    # disarmed after one use: a second call must not re-record (elapsed time unchanged)
+    capi.rmsnorm_backward(d["grad"], d["x"], d["weight"], rstd)
+    torch.cuda.synchronize()
+    ms2 = ctypes.c_float()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms2), ev[0], ev[1]) == 0 and ms2.value == ms.value
+    for e in ev:
+        hip.hipEventDestroy(e)
