@@ -69,10 +69,27 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     const int64_t b = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
 
-    u32x4 tr[CHUNKS], hr[CHUNKS];
-    load_one_plus_scale<T, C>(tr, scale + b * C, l);
+    // This sample's modulation row, staged once per workgroup through LDS: each thread
+    // forms t = rnd(1 + scale) for its share of the 16-byte pieces, then every lane picks up
+    // the pieces of its own columns.  (One-shot wavefronts would otherwise each repeat the
+    // whole row: 12 loads and ~120 VALU instructions per 6 KiB of useful traffic.)
+    constexpr int kPieces = C / VEC;  // 16-byte pieces per parameter row
+    __shared__ u32x4 lds_t[kPieces], lds_h[kPieces];
+    for (int i = threadIdx.x; i < kPieces; i += kRowThreads) {
+        float v[VEC];
+        E::unpack(load16(reinterpret_cast<const u32x4 *>(scale + b * C) + i), v);
 #pragma unroll
-    for (int k = 0; k < CHUNKS; ++k) hr[k] = load16(reinterpret_cast<const u32x4 *>(shift + b * C) + k * LANES + l);
+        for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
+        lds_t[i] = E::pack(v);
+        lds_h[i] = load16(reinterpret_cast<const u32x4 *>(shift + b * C) + i);
+    }
+    __syncthreads();
+    u32x4 tr[CHUNKS], hr[CHUNKS];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+        tr[k] = lds_t[k * LANES + l];
+        hr[k] = lds_h[k * LANES + l];
+    }
 
     const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
@@ -90,10 +107,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float v[VEC];
-            E::unpack(xr[k], v);
+            if constexpr (kIsBf16<T>) {  // row sum straight from the packed pairs
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) s += v[j];
+                for (int i = 0; i < 4; ++i) s = dot2_bf16(xr[k][i], kBf16OnesPair, s);
+            } else {
+                float v[VEC];
+                E::unpack(xr[k], v);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) s += v[j];
+            }
         }
         const float mu = group_sum<LANES>(s) / (float)C;
         float q = 0.0f;
@@ -113,6 +135,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             rstd[row] = r;
         }
 
+        const float nmr = -(mu * r);
         u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
         u32x4 *pn = WRITE_XNORM ? reinterpret_cast<u32x4 *>(xnorm + row * C) + l : nullptr;
 #pragma unroll
@@ -122,7 +145,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::unpack(tr[k], tv);
             E::unpack(hr[k], hv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] = (v[j] - mu) * r;
+            for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r as x*r + (-mu*r)
             if constexpr (WRITE_XNORM) {
                 const u32x4 xn = E::pack(v);
                 if (ok) store16_stream(pn + k * LANES, xn);
