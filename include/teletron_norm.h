@@ -22,6 +22,8 @@
  *     the caller (query the size first); the library never allocates.
  *
  * All pointers are device pointers, 16-byte aligned, row-major contiguous.
+ * Zero rows is a valid input: forward does nothing, backward writes zeros to the
+ * parameter gradients (no scratch needed); negative sizes are TT_NORM_EINVAL.
  * All calls are asynchronous on `stream` (a hipStream_t passed as void*;
  * NULL = the null stream).  Nothing here synchronises.
  */
@@ -39,7 +41,7 @@ extern "C" {
 
 enum tt_norm_status {
     TT_NORM_OK = 0,
-    TT_NORM_EINVAL = 1,       /* null pointer, non-positive size, rows not divisible by batch */
+    TT_NORM_EINVAL = 1,       /* null pointer, negative size, non-positive cols or batch */
     TT_NORM_EUNSUPPORTED = 2, /* cols or dtype the kernels are not built for */
     TT_NORM_EALIGN = 3,       /* a tensor pointer is not 16-byte aligned */
     TT_NORM_EWORKSPACE = 4,   /* workspace missing or smaller than *_workspace_bytes() */

@@ -32,6 +32,11 @@
 #ifndef TTN_ADALN_FWD_DYN_LDS
 #define TTN_ADALN_FWD_DYN_LDS 0
 #endif
+// Backward row fetch: all of g's accesses, then all of x's (two contiguous 6 KiB runs per
+// wavefront at 3072 columns) rather than alternating 1 KiB pieces; worth ~0.7 %.
+#ifndef TTN_BWD_LOAD_RUNS
+#define TTN_BWD_LOAD_RUNS 1
+#endif
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
@@ -217,11 +222,18 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         b.row = smp * rows_per_sample + rs;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
+#if TTN_BWD_LOAD_RUNS
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+#else
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
+#endif
         b.r = b.ok ? rstd[b.row] : 0.0f;
         b.mu = (!FROM_XNORM && b.ok) ? mean[b.row] : 0.0f;
     };
@@ -320,6 +332,7 @@ struct AdalnArgs {
 template <typename T, int C, bool WRITE_XNORM>
 static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, const void *x,
                            const void *scale, const void *shift, const AdalnArgs &a) {
+    if (a.rows_per_sample == 0) return TT_NORM_OK;  // empty input: nothing to do
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -344,6 +357,8 @@ template <typename T, int C, bool FROM_XNORM>
 static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g, const void *xin,
                             const void *scale, const float *mean, const float *rstd, int dtype,
                             void *ws, size_t ws_bytes, const AdalnArgs &a) {
+    // empty input: dscale/dshift are empty sums, written by the reducer over zero partial rows
+    if (a.rows_per_sample == 0) return launch_colreduce(dscale, dshift, nullptr, a.batch, 0, C, 2 * C, dtype, a.stream);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -366,12 +381,13 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
 
 static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sample, int64_t cols,
                             int dtype, std::initializer_list<const void *> ptrs) {
-    if (batch <= 0 || rows_per_sample <= 0 || cols <= 0)
+    if (batch <= 0 || rows_per_sample < 0 || cols <= 0)
         return fail(TT_NORM_EINVAL, "%s: batch=%lld rows_per_sample=%lld cols=%lld", who, (long long)batch,
                     (long long)rows_per_sample, (long long)cols);
     if (!tt_norm_supported(cols, dtype))
         return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
                     (long long)cols, dtype);
+    if (rows_per_sample == 0) return TT_NORM_OK;  // empty input: nothing is dereferenced
     for (const void *p : ptrs) {
         if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
         if (!aligned16(p)) return fail(TT_NORM_EALIGN, "%s: pointer %p not 16-byte aligned", who, p);
@@ -401,7 +417,7 @@ int tt_adaln_forward(void *out, float *mean, float *rstd, const void *x, const v
                      double eps, int dtype, void *stream) {
     int st = check_adaln_args("tt_adaln_forward", batch, rows_per_sample, cols, dtype, {out, x, scale, shift});
     if (st != TT_NORM_OK) return st;
-    if (!mean || !rstd) return fail(TT_NORM_EINVAL, "tt_adaln_forward: null mean/rstd");
+    if ((!mean || !rstd) && rows_per_sample > 0) return fail(TT_NORM_EINVAL, "tt_adaln_forward: null mean/rstd");
     const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
 #define CALL(T, C) return adaln_forward_t<T, C, false>(out, nullptr, mean, rstd, x, scale, shift, a)
     TTN_DISPATCH(dtype, cols, CALL);
@@ -414,7 +430,7 @@ int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x, 
     int st = check_adaln_args("tt_adaln_forward_xnorm", batch, rows_per_sample, cols, dtype,
                               {out, x_norm, x, scale, shift});
     if (st != TT_NORM_OK) return st;
-    if (!rstd) return fail(TT_NORM_EINVAL, "tt_adaln_forward_xnorm: null rstd");
+    if (!rstd && rows_per_sample > 0) return fail(TT_NORM_EINVAL, "tt_adaln_forward_xnorm: null rstd");
     const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
 #define CALL(T, C) return adaln_forward_t<T, C, true>(out, x_norm, nullptr, rstd, x, scale, shift, a)
     TTN_DISPATCH(dtype, cols, CALL);
@@ -438,7 +454,7 @@ int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, co
                       size_t workspace_bytes, void *stream) {
     int st = check_adaln_args("tt_adaln_backward", batch, rows_per_sample, cols, dtype, {dx, dout, x, scale});
     if (st != TT_NORM_OK) return st;
-    if (!dscale || !dshift || !mean || !rstd)
+    if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward: null dscale/dshift/mean/rstd");
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
 #define CALL(T, C)                                                                                \
@@ -455,7 +471,7 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
     int st = check_adaln_args("tt_adaln_backward_from_xnorm", batch, rows_per_sample, cols, dtype,
                               {dx, dout, x_norm, scale});
     if (st != TT_NORM_OK) return st;
-    if (!dscale || !dshift || !rstd)
+    if (!dscale || !dshift || (!rstd && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward_from_xnorm: null dscale/dshift/rstd");
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
 #define CALL(T, C)                                                                                 \

@@ -14,7 +14,7 @@ struct AdalnShape {
 };
 
 static AdalnShape adaln_shape(const torch::Tensor &x, const torch::Tensor &scale, int64_t rows, int64_t cols) {
-    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    TORCH_CHECK(rows >= 0 && cols > 0, "rows must be non-negative and cols positive");
     TORCH_CHECK(scale.numel() > 0 && scale.numel() % cols == 0, "scale has ", scale.numel(),
                 " elements, not a multiple of cols=", cols);
     const int64_t batch = scale.numel() / cols;
@@ -87,7 +87,7 @@ static void adaln_backward_impl(torch::Tensor &dinp, torch::Tensor &dscale, torc
     }
     c10::DeviceGuard guard(dev);
     const size_t need = tt_adaln_backward_workspace_bytes(s.batch, s.rows_per_sample, cols, s.dt);
-    TORCH_CHECK(need > 0, "unsupported AdaLN shape: cols=", cols);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported AdaLN shape: cols=", cols);
     at::Tensor ws = scratch(need, dout);
     if (mean)
         raise_on(tt_adaln_backward(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(),

@@ -18,7 +18,7 @@ void torch_launch_rms_forward(torch::Tensor &output, const torch::Tensor &input,
     check_dense_on(weight, dev, "weight");
     check_dense_on(inv_variance, dev, "inv_variance");
     const int dt = dtype_code(input, "input");
-    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    TORCH_CHECK(rows >= 0 && cols > 0, "rows must be non-negative and cols positive");
     check_elems(input, rows * cols, input.scalar_type(), "input");
     check_elems(output, rows * cols, input.scalar_type(), "output");
     check_elems(weight, cols, input.scalar_type(), "weight");
@@ -41,7 +41,7 @@ static void rms_backward_impl(torch::Tensor &dinp, torch::Tensor &dweight, const
     check_dense_on(weight, dev, "weight");
     check_dense_on(inv_variance, dev, "inv_variance");
     const int dt = dtype_code(dout, "dout");
-    TORCH_CHECK(rows > 0 && cols > 0, "rows and cols must be positive");
+    TORCH_CHECK(rows >= 0 && cols > 0, "rows must be non-negative and cols positive");
     check_elems(dout, rows * cols, dout.scalar_type(), "dout");
     check_elems(dinp, rows * cols, dout.scalar_type(), "dinp");
     check_elems(saved, rows * cols, dout.scalar_type(), saved_is_output ? "x_norm" : "input");
@@ -50,7 +50,7 @@ static void rms_backward_impl(torch::Tensor &dinp, torch::Tensor &dweight, const
     check_elems(inv_variance, rows, at::kFloat, "inv_variance");
     c10::DeviceGuard guard(dev);
     const size_t need = tt_rmsnorm_backward_workspace_bytes(rows, cols, dt);
-    TORCH_CHECK(need > 0, "unsupported RMSNorm shape: cols=", cols);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported RMSNorm shape: cols=", cols);
     at::Tensor ws = scratch(need, dout);
     auto fn = saved_is_output ? tt_rmsnorm_backward_from_out : tt_rmsnorm_backward;
     raise_on(fn(dinp.data_ptr(), dweight.data_ptr(), dout.data_ptr(), saved.data_ptr(), weight.data_ptr(),
@@ -103,7 +103,6 @@ void torch_launch_rms_forward_strided(torch::Tensor &output, const torch::Tensor
     const int64_t cols = weight.numel();
     const View3 v = view3(input, cols, "input");
     const int64_t rows = v.n[0] * v.n[1] * v.n[2];
-    TORCH_CHECK(rows > 0, "input is empty");
     check_elems(output, rows * cols, input.scalar_type(), "output");
     check_elems(weight, cols, input.scalar_type(), "weight");
     check_elems(inv_variance, rows, at::kFloat, "inv_variance");
@@ -131,7 +130,6 @@ void torch_launch_rms_backward_strided(torch::Tensor &dinp, torch::Tensor &dweig
     const View3 vd = view3(dinp, cols, "dinp");
     TORCH_CHECK(input.sizes() == dinp.sizes(), "dinp must have input's shape");
     const int64_t rows = vx.n[0] * vx.n[1] * vx.n[2];
-    TORCH_CHECK(rows > 0, "input is empty");
     TORCH_CHECK(input.scalar_type() == dout.scalar_type() && dinp.scalar_type() == dout.scalar_type(),
                 "input, dinp and dout must share a dtype");
     check_elems(dout, rows * cols, dout.scalar_type(), "dout");
@@ -140,7 +138,7 @@ void torch_launch_rms_backward_strided(torch::Tensor &dinp, torch::Tensor &dweig
     check_elems(inv_variance, rows, at::kFloat, "inv_variance");
     c10::DeviceGuard guard(dev);
     const size_t need = tt_rmsnorm_backward_workspace_bytes(rows, cols, dt);
-    TORCH_CHECK(need > 0, "unsupported RMSNorm shape: cols=", cols);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported RMSNorm shape: cols=", cols);
     at::Tensor ws = scratch(need, dout);
     raise_on(tt_rmsnorm_backward_strided(dinp.data_ptr(), dweight.data_ptr(), dout.data_ptr(), input.data_ptr(),
                                          weight.data_ptr(), inv_variance.data_ptr<float>(), vx.n[0], vx.n[1],

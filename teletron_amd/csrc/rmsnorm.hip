@@ -27,6 +27,11 @@
 #ifndef TTN_RMS_FWD_DYN_LDS
 #define TTN_RMS_FWD_DYN_LDS (C >= 1024 && sizeof(T) == 2 ? 51200 : 0)
 #endif
+// Backward row fetch: all of g's accesses, then all of x's (two contiguous 6 KiB runs per
+// wavefront at 3072 columns) rather than alternating 1 KiB pieces; worth ~0.7 %.
+#ifndef TTN_BWD_LOAD_RUNS
+#define TTN_BWD_LOAD_RUNS 1
+#endif
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
@@ -201,11 +206,18 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         b.doff = at.doff;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
+#if TTN_BWD_LOAD_RUNS
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+#else
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
+#endif
         b.r = b.ok ? rstd[at.row] : 0.0f;
     };
     auto process = [&](const RowRegs &b, auto &&between_passes) {
@@ -289,6 +301,7 @@ struct RmsTune {
 template <typename T, int C, typename Map>
 static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *w, const Map &map,
                              int64_t rows, double eps, hipStream_t stream) {
+    if (rows == 0) return TT_NORM_OK;  // empty input: nothing to do
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -313,6 +326,8 @@ template <typename T, int C, bool FROM_OUT, typename Map>
 static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin, const void *w,
                               const float *rstd, const Map &map, int64_t rows, int dtype, void *ws,
                               size_t ws_bytes, hipStream_t stream) {
+    // empty input: dweight is the empty sum, written by the reducer over zero partial rows
+    if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, 1, 0, C, C, dtype, stream);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -332,10 +347,11 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
 
 static int check_rms_args(const char *who, int64_t rows, int64_t cols, int dtype,
                           std::initializer_list<const void *> ptrs) {
-    if (rows <= 0 || cols <= 0) return fail(TT_NORM_EINVAL, "%s: rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
+    if (rows < 0 || cols <= 0) return fail(TT_NORM_EINVAL, "%s: rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
     if (!tt_norm_supported(cols, dtype))
         return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
                     (long long)cols, dtype);
+    if (rows == 0) return TT_NORM_OK;  // empty input: nothing is dereferenced
     for (const void *p : ptrs) {
         if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
         if (!aligned16(p)) return fail(TT_NORM_EALIGN, "%s: pointer %p not 16-byte aligned", who, p);
@@ -364,7 +380,7 @@ int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight
                        int64_t cols, double eps, int dtype, void *stream) {
     int st = check_rms_args("tt_rmsnorm_forward", rows, cols, dtype, {out, x, weight});
     if (st != TT_NORM_OK) return st;
-    if (!rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward: null rstd");
+    if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward: null rstd");
 #define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, DenseRows{rows}, rows, eps, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
@@ -385,7 +401,7 @@ int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x
                         size_t workspace_bytes, void *stream) {
     int st = check_rms_args("tt_rmsnorm_backward", rows, cols, dtype, {dx, dout, x, weight});
     if (st != TT_NORM_OK) return st;
-    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
+    if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
 #define CALL(T, C)                                                                                  \
     return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, DenseRows{rows}, rows, dtype, \
                                            workspace, workspace_bytes, (hipStream_t)stream)
@@ -398,7 +414,7 @@ int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, cons
                                  int dtype, void *workspace, size_t workspace_bytes, void *stream) {
     int st = check_rms_args("tt_rmsnorm_backward_from_out", rows, cols, dtype, {dx, dout, out, weight});
     if (st != TT_NORM_OK) return st;
-    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_from_out: null dweight/rstd");
+    if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_from_out: null dweight/rstd");
 #define CALL(T, C)                                                                                   \
     return rmsnorm_backward_t<T, C, true>(dx, dweight, dout, out, weight, rstd, DenseRows{rows}, rows, dtype, \
                                           workspace, workspace_bytes, (hipStream_t)stream)
@@ -408,7 +424,7 @@ int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, cons
 
 static int check_strided(const char *who, int64_t n0, int64_t n1, int64_t n2, int64_t cols, int dtype,
                          const int64_t (&strides)[3], const char *what) {
-    if (n0 <= 0 || n1 <= 0 || n2 <= 0)
+    if (n0 < 0 || n1 < 0 || n2 < 0)
         return fail(TT_NORM_EINVAL, "%s: sizes [%lld, %lld, %lld]", who, (long long)n0, (long long)n1, (long long)n2);
     if (!tt_norm_supported(cols, dtype)) return TT_NORM_OK;  // reported by the common check
     const int64_t vec = dtype == TT_NORM_BF16 ? 8 : 4;
@@ -428,7 +444,7 @@ int tt_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void
     const int64_t rows = n0 * n1 * n2;
     st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight});
     if (st != TT_NORM_OK) return st;
-    if (!rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward_strided: null rstd");
+    if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward_strided: null rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, 0, 0, 0};
 #define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, map, rows, eps, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
@@ -447,7 +463,7 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
     const int64_t rows = n0 * n1 * n2;
     st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight});
     if (st != TT_NORM_OK) return st;
-    if (!dweight || !rstd) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_strided: null dweight/rstd");
+    if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_strided: null dweight/rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, dxs0, dxs1, dxs2};
 #define CALL(T, C)                                                                                       \
     return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, map, rows, dtype, workspace, \

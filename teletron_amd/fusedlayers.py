@@ -68,6 +68,12 @@ def _require_gpu(t: torch.Tensor, what: str):
         raise ValueError(f"{what}: fused kernels need a GPU tensor, got device {t.device}")
 
 
+def _aligned_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned (a contiguous slice may start at any element)."""
+    t = t.contiguous()
+    return t.clone() if t.data_ptr() % 16 else t
+
+
 class FP32LayerNorm(nn.LayerNorm):
     """LayerNorm evaluated in fp32 and cast back (dit_fusedlayers.py:48-57)."""
 
@@ -89,10 +95,10 @@ class AdaLNModelFunction(Function):
     def forward(ctx, x, scale, shift, epsilon, cols):
         ext = _require_extension(fused_adaln, "fused_adaln")
         _require_gpu(x, "AdaLNModelFunction")
-        x = x.contiguous()
+        x = _aligned_contiguous(x)
         scale_c = scale.contiguous()
         shift_c = shift.contiguous()
-        if cols not in SUPPORTED_COLS or x.numel() == 0 or x.numel() % cols != 0:
+        if cols not in SUPPORTED_COLS or x.numel() % cols != 0:
             raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols} "
                              f"or unsupported cols (supported: {SUPPORTED_COLS})")
         rows = x.numel() // cols
@@ -116,7 +122,7 @@ class AdaLNModelFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         x, scale_c, mean, invvar = ctx.saved_tensors
-        grad_output = grad_output.contiguous()
+        grad_output = _aligned_contiguous(grad_output)
         if grad_output.dtype != x.dtype:
             grad_output = grad_output.to(x.dtype)
         grad_input = torch.empty_like(x)
@@ -280,14 +286,14 @@ class RMSNormModelFunction(Function):
     def forward(ctx, x, weight, epsilon, cols):
         ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
         _require_gpu(x, "RMSNormModelFunction")
-        if cols not in SUPPORTED_COLS or x.numel() == 0 or x.numel() % cols != 0:
+        if cols not in SUPPORTED_COLS or x.numel() % cols != 0:
             raise ValueError(f"Input size {x.numel()} not divisible by cols {cols} or unsupported cols value "
                              f"(supported: {SUPPORTED_COLS})")
         if weight.numel() != cols:
             raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
         strided = x.shape[-1] == cols and _strided_rows_ok(x)
         if not strided:
-            x = x.contiguous()
+            x = _aligned_contiguous(x)
         w = weight.contiguous()
         if w.dtype != x.dtype:
             w = w.to(x.dtype)
@@ -306,7 +312,7 @@ class RMSNormModelFunction(Function):
     @staticmethod
     def backward(ctx, grad_output):
         x, w, invvar = ctx.saved_tensors
-        grad_output = grad_output.contiguous()
+        grad_output = _aligned_contiguous(grad_output)
         if grad_output.dtype != x.dtype:
             grad_output = grad_output.to(x.dtype)
         grad_weight = torch.empty_like(w)

@@ -238,3 +238,30 @@ def test_rmsnorm_function_reads_qkv_view_in_place(FL, gpu_device):
     assert got[2][..., 2 * D:].abs().max() == 0
     # dweight sums two accumulated calls in bf16 on both sides: allow one extra bf16 rounding
     assert O.frac_outside(got[3].cpu(), want[3], 2e-2, 1e-3) == 0.0
+
+
+def test_empty_and_unaligned_inputs(FL, gpu_device):
+    """Zero rows: forward returns an empty tensor, backward returns zero parameter gradients.
+    A contiguous slice that starts at an odd element is copied to an aligned buffer, not rejected."""
+    w = torch.ones(128, device=gpu_device, dtype=torch.bfloat16, requires_grad=True)
+    x = torch.zeros(0, 24, 128, device=gpu_device, dtype=torch.bfloat16, requires_grad=True)
+    out = FL.RMSNormModelFunction.apply(x, w, EPS, 128)
+    assert out.shape == (0, 24, 128)
+    out.sum().backward()
+    assert x.grad.shape == x.shape and torch.count_nonzero(w.grad) == 0
+    sc = torch.zeros(2, 3072, device=gpu_device, dtype=torch.bfloat16, requires_grad=True)
+    sh = torch.zeros(2, 3072, device=gpu_device, dtype=torch.bfloat16, requires_grad=True)
+    xe = torch.zeros(2, 0, 3072, device=gpu_device, dtype=torch.bfloat16, requires_grad=True)
+    oe = FL.AdaLNModelFunction.apply(xe, sc, sh, EPS, 3072)
+    assert oe.shape == (2, 0, 3072)
+    oe.sum().backward()
+    assert torch.count_nonzero(sc.grad) == 0 and torch.count_nonzero(sh.grad) == 0
+
+    d = O.make_rmsnorm_inputs((33,), 128, torch.bfloat16, seed=60)
+    flat = torch.zeros(33 * 128 + 1, dtype=torch.bfloat16, device=gpu_device)
+    flat[1:] = d["x"].to(gpu_device).reshape(-1)
+    x_odd = flat[1:].view(33, 128)                  # contiguous, but starts 2 bytes into the allocation
+    assert x_odd.is_contiguous() and x_odd.data_ptr() % 16 != 0
+    got = FL.RMSNormModelFunction.apply(x_odd, d["weight"].to(gpu_device), EPS, 128)
+    want = O.eager_rmsnorm(d["x"], d["weight"], EPS)
+    fwd_ok(got, want, O.rmsnorm_excuse(want))

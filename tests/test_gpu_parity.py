@@ -319,7 +319,8 @@ def test_error_statuses(capi, gpu_device):
     assert L.tt_rmsnorm_forward(vp(x, 2), vp(r), vp(x), vp(w), 4, 3072, 1e-6, 0, None) == 3
     # null pointer / bad sizes
     assert L.tt_rmsnorm_forward(None, vp(r), vp(x), vp(w), 8, 3072, 1e-6, 0, None) == 1
-    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), 0, 3072, 1e-6, 0, None) == 1
+    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), -1, 3072, 1e-6, 0, None) == 1
+    assert L.tt_rmsnorm_forward(vp(x), vp(r), vp(x), vp(w), 0, 3072, 1e-6, 0, None) == 0   # zero rows: valid no-op
     # workspace too small
     need = L.tt_rmsnorm_backward_workspace_bytes(8, 3072, 0)
     assert need > 0

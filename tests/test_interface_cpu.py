@@ -138,3 +138,13 @@ def test_fp32_layer_norm():
     ln = FL.FP32LayerNorm(64, elementwise_affine=False, bias=False)
     want = torch.nn.functional.layer_norm(x.float(), (64,), None, None, ln.eps).bfloat16()
     assert torch.equal(ln(x), want)
+
+
+def test_c_abi_accepts_zero_rows_without_a_gpu_launch():
+    from teletron_amd import capi
+    L = capi.lib()
+    # forward over zero rows is a no-op: returns OK without touching any pointer
+    assert L.tt_rmsnorm_forward(None, None, None, None, 0, 3072, 1e-6, 0, None) == 0
+    assert L.tt_adaln_forward(None, None, None, None, None, None, 3, 0, 3072, 1e-6, 0, None) == 0
+    assert L.tt_rmsnorm_forward(None, None, None, None, -1, 3072, 1e-6, 0, None) == 1
+    assert L.tt_rmsnorm_backward_workspace_bytes(0, 3072, 0) == 0
