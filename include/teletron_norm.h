@@ -158,6 +158,39 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                  int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* ----------------------------------------------- gated residual + AdaLN
+ * The transformer blocks update the residual stream and then normalise it:
+ *     h2  = round(h + round(attn * gate[b]))
+ *     out = AdaLN(h2; scale[b], shift[b])
+ * (teletron/models/dit/dit_layerspec.py:152-167 in the double-stream block; the
+ * single-stream block ends with the same update, :351-352, feeding the next block's
+ * norm).  The reference runs these as separate elementwise kernels plus the norm; here
+ * one pass reads h and attn and writes h2 and out, and one backward pass produces every
+ * gradient.  h, attn, h2, out [batch * rows_per_sample, cols]; gate, scale, shift
+ * [batch, cols]; cols must be 3072.
+ */
+
+int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rstd,
+                                    const void *h, const void *attn, const void *gate,
+                                    const void *scale, const void *shift,
+                                    int64_t batch, int64_t rows_per_sample, int64_t cols,
+                                    double eps, int dtype, void *stream);
+
+size_t tt_gated_residual_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample,
+                                                        int64_t cols, int dtype);
+
+/* dout is the gradient of `out`; dh2 the gradient reaching h2 through its other uses
+ * (the residual stream continues past the norm), or NULL when there is none.
+ * Writes dh (gradient of h, = total gradient of h2), dattn = round(dh * gate[b])
+ * [rows, cols] and dgate = sum_rows round(dh * attn), dscale, dshift [batch, cols].
+ * mean, rstd are what the forward wrote; h2 is the forward's first output. */
+int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift,
+                                     const void *dout, const void *dh2, const void *h2,
+                                     const void *attn, const void *gate, const void *scale,
+                                     const float *mean, const float *rstd,
+                                     int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------- measurement
  * Arms a pair of HIP events (hipEvent_t passed as void*, created by the caller with
  * timing enabled) for the NEXT row kernel launched from this thread: `start` is

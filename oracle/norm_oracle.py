@@ -11,6 +11,11 @@ when its fused kernels are off -- the behaviour the fused kernels must match:
   * AdaLN    -- teletron/models/dit/dit_fusedlayers.py:198,223 (and :251,271)
         out = LayerNorm(C, elementwise_affine=False, eps)(x) * (1 + scale[:, None]) + shift[:, None]
 
+  * gated residual + AdaLN -- teletron/models/dit/dit_layerspec.py:152,158,161-163
+        h2  = h + attn * gate.unsqueeze(1)
+        out = LayerNorm(C, elementwise_affine=False, eps)(h2) * (1 + scale[:, None]) + shift[:, None]
+    (h2 also continues as the residual stream, :180-182)
+
 Three layers of the same math live here, each one a check on the others:
 
   eager_*     the formulas above, verbatim in behaviour, differentiated by
@@ -76,6 +81,26 @@ def eager_adaln_fwd_bwd(x, scale, shift, grad, eps: float = EPS):
     return out.detach(), x.grad, scale.grad, shift.grad
 
 
+def eager_gated_residual_adaln(h, attn, gate, scale, shift, eps: float = EPS):
+    """dit_layerspec.py:152 then :158,:161-163.  h, attn [B,S,C]; gate, scale, shift [B,C].
+    Returns (h2, out): the updated residual stream and its modulated norm."""
+    h2 = h + attn * gate.unsqueeze(1)
+    return h2, eager_adaln(h2, scale, shift, eps)
+
+
+def eager_gated_residual_adaln_fwd_bwd(h, attn, gate, scale, shift, grad_out, grad_h2=None,
+                                       eps: float = EPS):
+    """Returns (h2, out, dh, dattn, dgate, dscale, dshift) as autograd produces them;
+    grad_h2 is the gradient h2 receives from its later uses (None: it has none)."""
+    leaves = [t.detach().clone().requires_grad_(True) for t in (h, attn, gate, scale, shift)]
+    h2, out = eager_gated_residual_adaln(*leaves, eps)
+    if grad_h2 is None:
+        out.backward(grad_out)
+    else:
+        torch.autograd.backward([out, h2], [grad_out, grad_h2])
+    return (h2.detach(), out.detach()) + tuple(t.grad for t in leaves)
+
+
 # --------------------------------------------------------------------------
 # staged: every rounding point written out (what a fused kernel must follow)
 # --------------------------------------------------------------------------
@@ -139,9 +164,37 @@ def staged_adaln_bwd(x, scale, mean, rstd, grad):
     return dx, dscale, dshift
 
 
+def staged_gated_residual_adaln_fwd(h, attn, gate, scale, shift, eps: float = EPS):
+    """Returns (h2, out, mean, rstd).  Rounding points: m = attn*gate; h2 = h+m; then the AdaLN chain."""
+    m = attn * gate[:, None]
+    h2 = h + m
+    out, mean, rstd = staged_adaln_fwd(h2, scale, shift, eps)
+    return h2, out, mean, rstd
+
+
+def staged_gated_residual_adaln_bwd(h2, attn, gate, scale, mean, rstd, grad_out, grad_h2=None):
+    """dxl = AdaLN dx (rounded); dh = round(dxl + grad_h2); dattn = round(dh*gate);
+    dgate = sum_s round(dh*attn).  Returns (dh, dattn, dgate, dscale, dshift)."""
+    dxl, dscale, dshift = staged_adaln_bwd(h2, scale, mean, rstd, grad_out)
+    dh = dxl if grad_h2 is None else dxl + grad_h2
+    dattn = dh * gate[:, None]
+    dgate = (dh * attn).sum(1).to(gate.dtype)
+    return dh, dattn, dgate, dscale, dshift
+
+
 # --------------------------------------------------------------------------
 # truth: float64 closed forms, no intermediate rounding
 # --------------------------------------------------------------------------
+
+def truth_gated_residual_adaln_fwd_bwd(h, attn, gate, scale, shift, grad_out, grad_h2=None,
+                                       eps: float = EPS):
+    """Returns (h2, out, dh, dattn, dgate, dscale, dshift) in float64."""
+    hd, ad, qd = h.double(), attn.double(), gate.double()
+    h2 = hd + ad * qd[:, None]
+    out, dxl, dscale, dshift = truth_adaln_fwd_bwd(h2, scale, shift, grad_out, eps)
+    dh = dxl if grad_h2 is None else dxl + grad_h2.double()
+    return h2, out, dh, dh * qd[:, None], (dh * ad).sum(1), dscale, dshift
+
 
 def truth_rmsnorm_fwd_bwd(x, weight, grad, eps: float = EPS):
     C = x.shape[-1]
@@ -242,12 +295,31 @@ def adaln_excuse(x, scale, shift, want_out, eps: float = EPS) -> torch.Tensor:
     return p * 2.0 ** -6 + want_out.float().abs() * 2.0 ** -7
 
 
-def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float) -> float:
-    """Fraction of elements with |got-want| > atol + rtol*|want| (allclose's rule)."""
+def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float,
+                 magnitude: Optional[torch.Tensor] = None) -> float:
+    """Fraction of elements with |got-want| > atol + rtol*|want| (allclose's rule).
+    `magnitude`, when given, replaces |want| in the bound: for a result that is a sum of
+    separately rounded terms (h2's gradient = the norm's dx + the upstream gradient) the honest
+    scale of a one-ulp disagreement is the size of the terms, not of a sum that may cancel."""
     g, w = got.double().cpu(), want.double().cpu()
     if g.numel() == 0:
         return 0.0
-    return float(((g - w).abs() > atol + rtol * w.abs()).double().mean())
+    m = w.abs() if magnitude is None else magnitude.double().cpu().abs()
+    return float(((g - w).abs() > atol + rtol * m).double().mean())
+
+
+def colsum_outside(got: torch.Tensor, want: torch.Tensor, terms: torch.Tensor, dim: int,
+                   rtol: float = 1e-2, ulp: float = 2.0 ** -5) -> int:
+    """Number of column sums with |got-want| > rtol*|want| + ulp*||terms||_2, the L2 norm taken over
+    the summed dimension.  For a column sum whose TERMS are known to one rounding of the element
+    type only (each may differ by an ulp between two correct implementations): such errors add
+    like a random walk, so the column's L2 mass is their natural scale: a per-term error uniform
+    within one ulp (2^-8 relative) gives a sum error of about 2^-8 * 0.8 * L2 at one sigma, and
+    the eager result itself sits up to 2^-6 * L2 from the float64 truth over thousands of columns.
+    A dropped or misplaced term moves a column by the order of L2 itself."""
+    l2 = terms.double().cpu().pow(2).sum(dim).sqrt().reshape(want.shape)
+    g, w = got.double().cpu().reshape(want.shape), want.double().cpu()
+    return int(((g - w).abs() > rtol * w.abs() + ulp * l2).sum())
 
 
 # --------------------------------------------------------------------------
@@ -290,6 +362,24 @@ CONFIGS = {
     "cfg4_adaln_bf16": ("adaln", dict(batch=1, seq=118800, cols=3072, dtype=torch.bfloat16)),
     "cfg5_adaln_bf16": ("adaln", dict(batch=4, seq=11056, cols=3072, dtype=torch.bfloat16, sigma=2.0)),
 }
+
+
+def make_gated_inputs(batch: int, seq: int, cols: int, dtype: torch.dtype, seed: int = 0,
+                      with_grad_h2: bool = True):
+    """(h, attn, gate, scale, shift, grad_out, grad_h2): a residual stream of O(1) entries with a
+    per-row offset, attention output of O(1), gates and modulation of the size an adaLN-Zero linear
+    produces after some training (|.| ~ 0.3)."""
+    g = _gen(seed + 77)
+    h = torch.randn(batch, seq, cols, generator=g) * (0.5 + torch.rand(batch, seq, 1, generator=g) * 1.5) \
+        + torch.randn(batch, seq, 1, generator=g) * 0.3
+    attn = torch.randn(batch, seq, cols, generator=g)
+    gate = torch.randn(batch, cols, generator=g) * 0.3
+    scale = torch.randn(batch, cols, generator=g) * 0.3
+    shift = torch.randn(batch, cols, generator=g) * 0.3
+    grad_out = torch.randn(batch, seq, cols, generator=g) * 0.1
+    grad_h2 = torch.randn(batch, seq, cols, generator=g) * 0.1 if with_grad_h2 else None
+    cast = lambda t: None if t is None else t.to(dtype)
+    return tuple(cast(t) for t in (h, attn, gate, scale, shift, grad_out, grad_h2))
 
 
 def make_config_inputs(name: str, seed: int = 0, rows_limit: Optional[int] = None):

@@ -24,6 +24,8 @@ EXPORTS = (
     "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
     "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
     "tt_norm_profile_next_row_kernel",
+    "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
+    "tt_gated_residual_adaln_backward",
 )
 
 
@@ -61,6 +63,10 @@ def lib() -> ctypes.CDLL:
         L.tt_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
         L.tt_adaln_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_from_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
+        L.tt_gated_residual_adaln_forward.argtypes = [vp] * 9 + [i64, i64, i64, dbl, ci, vp]
+        L.tt_gated_residual_adaln_backward_workspace_bytes.restype = sz
+        L.tt_gated_residual_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
+        L.tt_gated_residual_adaln_backward.argtypes = [vp] * 13 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
         L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
@@ -222,6 +228,49 @@ def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False):
                                        _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n, _stream(x)),
                    "tt_adaln_backward")
     return dx, dscale, dshift
+
+
+def gated_residual_adaln_forward(h, attn, gate, scale, shift, eps: float):
+    """h2 = h + attn*gate[b]; out = AdaLN(h2).  Returns (h2, out, mean, rstd)."""
+    _dense_gpu(h, attn, gate, scale, shift)
+    cols = h.shape[-1]
+    batch = scale.numel() // cols
+    rows = h.numel() // cols
+    if rows % batch:
+        raise ValueError("rows not divisible by batch")
+    h2 = torch.empty_like(h)
+    out = torch.empty_like(h)
+    mean = torch.empty(rows, dtype=torch.float32, device=h.device)
+    rstd = torch.empty(rows, dtype=torch.float32, device=h.device)
+    with torch.cuda.device(h.device):
+        _check(lib().tt_gated_residual_adaln_forward(_p(h2), _p(out), _p(mean), _p(rstd), _p(h), _p(attn),
+                                                     _p(gate), _p(scale), _p(shift), batch, rows // batch, cols,
+                                                     eps, _dt(h), _stream(h)), "tt_gated_residual_adaln_forward")
+    return h2, out, mean, rstd
+
+
+def gated_residual_adaln_backward(dout, dh2, h2, attn, gate, scale, mean, rstd):
+    """Returns (dh, dattn, dgate, dscale, dshift); dh2 may be None."""
+    _dense_gpu(dout, h2, attn, gate, scale, mean, rstd)
+    if dh2 is not None:
+        _dense_gpu(dh2)
+    cols = h2.shape[-1]
+    batch = scale.numel() // cols
+    rows = h2.numel() // cols
+    dh = torch.empty_like(h2)
+    dattn = torch.empty_like(h2)
+    dgate = torch.empty_like(scale)
+    dscale = torch.empty_like(scale)
+    dshift = torch.empty_like(scale)
+    with torch.cuda.device(h2.device):
+        L = lib()
+        n = L.tt_gated_residual_adaln_backward_workspace_bytes(batch, rows // batch, cols, _dt(h2))
+        ws = _workspace(n, h2)
+        _check(L.tt_gated_residual_adaln_backward(_p(dh), _p(dattn), _p(dgate), _p(dscale), _p(dshift), _p(dout),
+                                                  _p(dh2), _p(h2), _p(attn), _p(gate), _p(scale), _p(mean),
+                                                  _p(rstd), batch, rows // batch, cols, _dt(h2), _p(ws), n,
+                                                  _stream(h2)), "tt_gated_residual_adaln_backward")
+    return dh, dattn, dgate, dscale, dshift
 
 
 def stream_copy(dst: torch.Tensor, src: torch.Tensor):

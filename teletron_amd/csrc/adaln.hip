@@ -59,10 +59,13 @@ __device__ __forceinline__ void load_one_plus_scale(u32x4 *tr, const T *__restri
     }
 }
 
-template <typename T, int C, bool WRITE_XNORM>
-__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 2) void adaln_fwd_kernel(
+// GATED = true: the normalised tensor is first formed as h2 = rnd(x + rnd(attn * gate[b])) (the
+// gated residual update that precedes the norm in the transformer blocks) and written out too.
+template <typename T, int C, bool WRITE_XNORM, bool GATED>
+__global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? (GATED ? 3 : 4) : 2) void adaln_fwd_kernel(
     T *__restrict__ out, T *__restrict__ xnorm, float *__restrict__ mean, float *__restrict__ rstd,
     const T *__restrict__ x, const T *__restrict__ scale, const T *__restrict__ shift,
+    T *__restrict__ h2_out, const T *__restrict__ attn, const T *__restrict__ gate,
     int64_t rows_per_sample, int blocks_per_sample, float eps) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     // the pieces of its own columns.  (One-shot wavefronts would otherwise each repeat the
     // whole row: 12 loads and ~120 VALU instructions per 6 KiB of useful traffic.)
     constexpr int kPieces = C / VEC;  // 16-byte pieces per parameter row
-    __shared__ u32x4 lds_t[kPieces], lds_h[kPieces];
+    __shared__ u32x4 lds_t[kPieces], lds_h[kPieces], lds_g[GATED ? kPieces : 1];
     for (int i = threadIdx.x; i < kPieces; i += kRowThreads) {
         float v[VEC];
         E::unpack(load16(reinterpret_cast<const u32x4 *>(scale + b * C) + i), v);
@@ -87,6 +90,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
         lds_t[i] = E::pack(v);
         lds_h[i] = load16(reinterpret_cast<const u32x4 *>(shift + b * C) + i);
+        if constexpr (GATED) lds_g[i] = load16(reinterpret_cast<const u32x4 *>(gate + b * C) + i);
     }
     __syncthreads();
     u32x4 tr[CHUNKS], hr[CHUNKS];
@@ -108,6 +112,27 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         u32x4 xr[CHUNKS];
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        if constexpr (GATED) {
+            const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + row * C) + l;
+            u32x4 *ph = reinterpret_cast<u32x4 *>(h2_out + row * C) + l;
+            u32x4 ar[CHUNKS];
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) ar[k] = ok ? load16_stream(pa + k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+                float hv[VEC], av[VEC], gv[VEC];
+                E::unpack(xr[k], hv);
+                E::unpack(ar[k], av);
+                E::unpack(lds_g[k * LANES + l], gv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) av[j] *= gv[j];
+                E::round(av);  // attn * gate materialised in the element type
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) hv[j] += av[j];
+                xr[k] = E::pack(hv);  // h2: the new residual stream, and the row that is normalised
+                if (ok) store16_stream(ph + k * LANES, xr[k]);
+            }
+        }
 
         float s = 0.0f;
 #pragma unroll
@@ -176,17 +201,26 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // flight while the current one is processed.  With xhat = x*r - mu*r the row
 // reductions reduce to sum_c gx and sum_c gx*x, both taken straight from packed
 // bf16 pairs, and dx becomes r*gx + x*K1 + K0 with per-row scalars K1, K0.
-template <typename T, int C, bool FROM_XNORM>
+//
+// GATED = true (gated residual + AdaLN): xin is the saved h2; the gradient of h2 is
+// dh = rnd(rnd(dx of the norm) + e) with e the gradient arriving at h2 from its other use (may be
+// absent), written to dx; additionally da = rnd(dh * gate[b]) is written and
+// dgate[b] += rnd(dh * attn) is accumulated as a third set of column sums.
+template <typename T, int C, bool FROM_XNORM, bool GATED>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void adaln_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
-    const float *__restrict__ rstd, int64_t rows_per_sample, int blocks_per_sample) {
+    const float *__restrict__ rstd, T *__restrict__ da, const T *__restrict__ e,
+    const T *__restrict__ attn, const T *__restrict__ gate, int64_t rows_per_sample,
+    int blocks_per_sample) {
+    static_assert(!(GATED && FROM_XNORM), "the gated form works from the saved h2");
+    constexpr int NSETS = GATED ? 3 : 2;
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
     // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
     constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_ADALN_BWD_ROW_BUFFERS;
-    __shared__ float lds[2 * C];
+    __shared__ float lds[NSETS * C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
     const int l = lane % LANES;
@@ -202,9 +236,19 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         for (int k = 0; k < CHUNKS; ++k) E::unpack(tr[k], tv[k]);
     }
 
-    float acc[2][CHUNKS][VEC];  // [0] = dscale, [1] = dshift
+    // gate[sample]: unpacked once for 2-byte elements; 4-byte rows have no registers to spare and
+    // re-read it (cache hits) where it is used
+    constexpr bool kGateResident = GATED && sizeof(T) == 2;
+    [[maybe_unused]] float gatev[kGateResident ? CHUNKS : 1][VEC];
+    if constexpr (kGateResident) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+        for (int k = 0; k < CHUNKS; ++k)
+            E::unpack(load16(reinterpret_cast<const u32x4 *>(gate + smp * C) + k * LANES + l), gatev[k]);
+    }
+
+    float acc[NSETS][CHUNKS][VEC];  // [0] = dscale, [1] = dshift, [2] = dgate
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s)
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
@@ -212,6 +256,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 
     struct RowRegs {
         u32x4 g[CHUNKS], x[CHUNKS];
+        u32x4 a[kGateResident ? CHUNKS : 1], e[kGateResident ? CHUNKS : 1];
         float r, mu;
         int64_t row;
         bool ok;
@@ -234,6 +279,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
 #endif
+        if constexpr (kGateResident) {  // 4-byte rows fetch these two where they are used instead
+            const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + b.row * C) + l;
+            const u32x4 *pe = reinterpret_cast<const u32x4 *>(e + b.row * C) + l;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.a[k] = b.ok ? load16_stream(pa + k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k)
+                b.e[k] = (b.ok && e != nullptr) ? load16_stream(pe + k * LANES) : u32x4{0, 0, 0, 0};
+        }
         b.r = b.ok ? rstd[b.row] : 0.0f;
         b.mu = (!FROM_XNORM && b.ok) ? mean[b.row] : 0.0f;
     };
@@ -291,7 +345,40 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 xn[j] = FROM_XNORM ? xv[j] : fmaf(xv[j], r, nmr);
                 acc[1][k][j] += gv[j];
             }
-            if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
+            if constexpr (GATED) {
+                float ev[VEC], av[VEC], dav[VEC];
+                E::round(o);  // the norm's dx, materialised in the element type
+                if constexpr (kGateResident) {
+                    E::unpack(b.e[k], ev);
+                    E::unpack(b.a[k], av);
+                } else {
+                    const int64_t at = b.row * (C / VEC) + l + k * LANES;
+                    const u32x4 zero{0, 0, 0, 0};
+                    E::unpack((b.ok && e != nullptr) ? load16_stream(reinterpret_cast<const u32x4 *>(e) + at) : zero, ev);
+                    E::unpack(b.ok ? load16_stream(reinterpret_cast<const u32x4 *>(attn) + at) : zero, av);
+                }
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o[j] += ev[j];
+                const u32x4 dhp = E::pack(o);  // dh: gradient of h2 = of the residual input
+                if (b.ok) store16_stream(pd + k * LANES, dhp);
+                E::unpack(dhp, o);
+                if constexpr (kGateResident) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) dav[j] = o[j] * gatev[k][j];
+                } else {
+                    E::unpack(load16(reinterpret_cast<const u32x4 *>(gate + smp * C) + k * LANES + l), dav);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) dav[j] *= o[j];
+                }
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) av[j] *= o[j];
+                if (b.ok) store16_stream(reinterpret_cast<u32x4 *>(da + b.row * C) + l + k * LANES, E::pack(dav));
+                E::round(av);  // dh*attn materialised in the element type before the column sum
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
+            } else {
+                if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
+            }
             if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
@@ -305,7 +392,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
     int64_t grp = (int64_t)slot * kRowWaves + wave;
     row_pipeline<kRowBuffers, TTN_ADALN_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
-    flush_column_partials<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds);
+    flush_column_partials<G, NSETS>(acc, partial + (int64_t)blockIdx.x * (NSETS * C), lds);
 }
 
 // Same launch policy as RMSNorm: forward one-shot at 3072 columns, backward one
@@ -329,9 +416,17 @@ struct AdalnArgs {
     hipStream_t stream;
 };
 
-template <typename T, int C, bool WRITE_XNORM>
+struct GatedPtrs {  // the extra operands of the gated-residual form (all null otherwise)
+    void *h2_or_da;    // forward: h2 out;   backward: da out
+    const void *e;     // backward: gradient arriving at h2 from its other use, or null
+    const void *attn;
+    const void *gate;
+};
+
+template <typename T, int C, bool WRITE_XNORM, bool GATED = false>
 static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, const void *x,
-                           const void *scale, const void *shift, const AdalnArgs &a) {
+                           const void *scale, const void *shift, const AdalnArgs &a,
+                           const GatedPtrs &gp = GatedPtrs{nullptr, nullptr, nullptr, nullptr}) {
     if (a.rows_per_sample == 0) return TT_NORM_OK;  // empty input: nothing to do
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
@@ -341,9 +436,10 @@ static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, con
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln forward: grid too large");
     {
         RowKernelProfile prof(a.stream);
-        adaln_fwd_kernel<T, C, WRITE_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
+        adaln_fwd_kernel<T, C, WRITE_XNORM, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
             (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
-            a.rows_per_sample, p.blocks_per_sample, (float)a.eps);
+            (T *)gp.h2_or_da, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample, p.blocks_per_sample,
+            (float)a.eps);
     }
     return check_launch("adaln forward launch");
 }
@@ -353,30 +449,34 @@ static RowPlan adaln_backward_plan(int64_t batch, int64_t rows_per_sample, int c
     return make_row_plan(batch, rows_per_sample, RowGeom<T, C>::RPW, AdalnTune<T, C>::kBwdBlocksPerCu, cus);
 }
 
-template <typename T, int C, bool FROM_XNORM>
+template <typename T, int C, bool FROM_XNORM, bool GATED = false>
 static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g, const void *xin,
                             const void *scale, const float *mean, const float *rstd, int dtype,
-                            void *ws, size_t ws_bytes, const AdalnArgs &a) {
-    // empty input: dscale/dshift are empty sums, written by the reducer over zero partial rows
-    if (a.rows_per_sample == 0) return launch_colreduce(dscale, dshift, nullptr, a.batch, 0, C, 2 * C, dtype, a.stream);
+                            void *ws, size_t ws_bytes, const AdalnArgs &a, void *dgate = nullptr,
+                            const GatedPtrs &gp = GatedPtrs{nullptr, nullptr, nullptr, nullptr}) {
+    constexpr int NSETS = GATED ? 3 : 2;
+    // empty input: the parameter gradients are empty sums, written by the reducer over zero partial rows
+    if (a.rows_per_sample == 0)
+        return launch_colreduce(dscale, dshift, dgate, nullptr, a.batch, 0, C, NSETS * C, dtype, a.stream);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
     const RowPlan p = adaln_backward_plan<T, C>(a.batch, a.rows_per_sample, cus);
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "adaln backward: grid too large");
-    const size_t need = (size_t)p.blocks * 2 * C * sizeof(float);
+    const size_t need = (size_t)p.blocks * NSETS * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
     {
         RowKernelProfile prof(a.stream);
-        adaln_bwd_kernel<T, C, FROM_XNORM><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+        adaln_bwd_kernel<T, C, FROM_XNORM, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
             (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
-            a.rows_per_sample, p.blocks_per_sample);
+            (T *)gp.h2_or_da, (const T *)gp.e, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample,
+            p.blocks_per_sample);
     }
     st = check_launch("adaln backward launch");
     if (st != TT_NORM_OK) return st;
-    return launch_colreduce(dscale, dshift, (const float *)ws, a.batch, p.blocks_per_sample, C, 2 * C,
-                            dtype, a.stream);
+    return launch_colreduce(dscale, dshift, dgate, (const float *)ws, a.batch, p.blocks_per_sample, C,
+                            NSETS * C, dtype, a.stream);
 }
 
 static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sample, int64_t cols,
@@ -479,6 +579,53 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                         workspace, workspace_bytes, a)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
+}
+
+/* ---- gated residual + AdaLN (3072 columns) ---- */
+
+int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h,
+                                    const void *attn, const void *gate, const void *scale,
+                                    const void *shift, int64_t batch, int64_t rows_per_sample,
+                                    int64_t cols, double eps, int dtype, void *stream) {
+    int st = check_adaln_args("tt_gated_residual_adaln_forward", batch, rows_per_sample, cols, dtype,
+                              {h2, out, h, attn, gate, scale, shift});
+    if (st != TT_NORM_OK) return st;
+    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_forward: built for cols 3072 only");
+    if ((!mean || !rstd) && rows_per_sample > 0)
+        return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_forward: null mean/rstd");
+    const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
+    const GatedPtrs gp{h2, nullptr, attn, gate};
+    if (dtype == TT_NORM_BF16)
+        return adaln_forward_t<bf16_t, 3072, false, true>(out, nullptr, mean, rstd, h, scale, shift, a, gp);
+    return adaln_forward_t<float, 3072, false, true>(out, nullptr, mean, rstd, h, scale, shift, a, gp);
+}
+
+size_t tt_gated_residual_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols,
+                                                        int dtype) {
+    // three sets of column sums (dscale, dshift, dgate) instead of two
+    return tt_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype) / 2 * 3;
+}
+
+int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift,
+                                     const void *dout, const void *dh2, const void *h2, const void *attn,
+                                     const void *gate, const void *scale, const float *mean,
+                                     const float *rstd, int64_t batch, int64_t rows_per_sample,
+                                     int64_t cols, int dtype, void *workspace, size_t workspace_bytes,
+                                     void *stream) {
+    int st = check_adaln_args("tt_gated_residual_adaln_backward", batch, rows_per_sample, cols, dtype,
+                              {dh, dattn, dout, h2, attn, gate, scale});
+    if (st != TT_NORM_OK) return st;
+    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_backward: built for cols 3072 only");
+    if (dh2 && !aligned16(dh2)) return fail(TT_NORM_EALIGN, "tt_gated_residual_adaln_backward: dh2 not 16-byte aligned");
+    if (!dgate || !dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
+        return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_backward: null dgate/dscale/dshift/mean/rstd");
+    const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
+    const GatedPtrs gp{dattn, dh2, attn, gate};
+    if (dtype == TT_NORM_BF16)
+        return adaln_backward_t<bf16_t, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
+                                                           workspace, workspace_bytes, a, dgate, gp);
+    return adaln_backward_t<float, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
+                                                      workspace, workspace_bytes, a, dgate, gp);
 }
 
 }  // extern "C"

@@ -119,7 +119,74 @@ void torch_launch_adaln_backward_x(torch::Tensor &dinp, torch::Tensor &dscale, t
     adaln_backward_impl(dinp, dscale, dshift, dout, input, scale, &mean, inv_variance, rows, cols);
 }
 
+// Gated residual update fused with the norm that follows it:
+// h2 = input + attn * gate[b];  output = AdaLN(h2).  No counterpart in the reference's module.
+void torch_launch_gated_adaln_forward(torch::Tensor &h2, torch::Tensor &output, const torch::Tensor &input,
+                                      const torch::Tensor &attn, const torch::Tensor &gate,
+                                      const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                      int64_t cols, double epsilon, torch::Tensor &mean,
+                                      torch::Tensor &inv_variance) {
+    const auto dev = input.device();
+    for (auto *t : {&h2, &output, &mean, &inv_variance}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&input, &attn, &gate, &scale, &shift}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(input, scale, rows, cols);
+    const auto st = input.scalar_type();
+    for (auto *t : {&input, &attn}) check_elems(*t, rows * cols, st, "input/attn");
+    check_elems(h2, rows * cols, st, "h2");
+    check_elems(output, rows * cols, st, "output");
+    for (auto *t : {&gate, &scale, &shift}) check_elems(*t, scale.numel(), st, "gate/scale/shift");
+    check_elems(mean, rows, at::kFloat, "mean");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_gated_residual_adaln_forward(h2.data_ptr(), output.data_ptr(), mean.data_ptr<float>(),
+                                             inv_variance.data_ptr<float>(), input.data_ptr(), attn.data_ptr(),
+                                             gate.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch,
+                                             s.rows_per_sample, cols, epsilon, s.dt, current_stream(input)),
+             "tt_gated_residual_adaln_forward");
+}
+
+// dh2: gradient reaching h2 from its other uses, or None.
+void torch_launch_gated_adaln_backward(torch::Tensor &dinp, torch::Tensor &dattn, torch::Tensor &dgate,
+                                       torch::Tensor &dscale, torch::Tensor &dshift, const torch::Tensor &dout,
+                                       const c10::optional<torch::Tensor> &dh2, const torch::Tensor &h2,
+                                       const torch::Tensor &attn, const torch::Tensor &gate,
+                                       const torch::Tensor &scale, const torch::Tensor &mean,
+                                       const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    const auto dev = dout.device();
+    for (auto *t : {&dinp, &dattn, &dgate, &dscale, &dshift}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&dout, &h2, &attn, &gate, &scale, &mean, &inv_variance}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(dout, scale, rows, cols);
+    const auto st = dout.scalar_type();
+    for (auto *t : {&dout, &h2, &attn}) check_elems(*t, rows * cols, st, "dout/h2/attn");
+    for (auto *t : {&dinp, &dattn}) check_elems(*t, rows * cols, st, "dinp/dattn");
+    for (auto *t : {&gate, &scale}) check_elems(*t, scale.numel(), st, "gate/scale");
+    for (auto *t : {&dgate, &dscale, &dshift}) check_elems(*t, scale.numel(), st, "dgate/dscale/dshift");
+    check_elems(mean, rows, at::kFloat, "mean");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    const void *dh2_ptr = nullptr;
+    if (dh2.has_value() && dh2->defined()) {
+        check_dense_on(*dh2, dev, "dh2");
+        check_elems(*dh2, rows * cols, st, "dh2");
+        dh2_ptr = dh2->data_ptr();
+    }
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_gated_residual_adaln_backward_workspace_bytes(s.batch, s.rows_per_sample, cols, s.dt);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported gated AdaLN shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    raise_on(tt_gated_residual_adaln_backward(dinp.data_ptr(), dattn.data_ptr(), dgate.data_ptr(),
+                                              dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(), dh2_ptr,
+                                              h2.data_ptr(), attn.data_ptr(), gate.data_ptr(), scale.data_ptr(),
+                                              mean.data_ptr<float>(), inv_variance.data_ptr<float>(), s.batch,
+                                              s.rows_per_sample, cols, s.dt, ws.data_ptr(), need,
+                                              current_stream(dout)),
+             "tt_gated_residual_adaln_backward");
+}
+
 PYBIND11_MODULE(fused_adaln, m) {
+    m.def("torch_launch_gated_adaln_forward", &torch_launch_gated_adaln_forward,
+          "gated residual update + AdaLN forward kernel");
+    m.def("torch_launch_gated_adaln_backward", &torch_launch_gated_adaln_backward,
+          "gated residual update + AdaLN backward kernel");
     m.def("torch_launch_adaln_forward", &torch_launch_adaln_forward, "AdaLN forward kernel");
     m.def("torch_launch_adaln_backward", &torch_launch_adaln_backward,
           "AdaLN backward kernel (from the saved normalised rows)");

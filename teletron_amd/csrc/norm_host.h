@@ -57,8 +57,9 @@ RowPlan make_row_plan(int64_t batch, int64_t rows_per_sample, int rows_per_wave,
                       int blocks_per_cu, int cus);
 
 // Stage-2 reducer: partial[batch][blocks_per_sample][ncols] fp32 ->
-// out0[batch][C] (columns [0, C)) and, when ncols == 2C, out1[batch][C].
-int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch,
+// out0[batch][C] (columns [0, C)), out1[batch][C] (columns [C, 2C)) when ncols >= 2C,
+// out2[batch][C] (columns [2C, 3C)) when ncols == 3C.
+int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, int64_t batch,
                      int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
                      hipStream_t stream);
 

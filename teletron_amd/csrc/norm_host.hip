@@ -79,7 +79,7 @@ RowPlan make_row_plan(int64_t batch, int64_t rows_per_sample, int rows_per_wave,
 }
 
 // ---- stage 2: fixed-order column reduction ---------------------------------
-// partial[b][g][ncols] -> out[b][c].  A workgroup of 32 x 32 threads owns 32
+// partial[b][g][ncols] -> out0/out1/out2[b][c] (ncols = 1, 2 or 3 sets of C columns).  A workgroup of 32 x 32 threads owns 32
 // adjacent columns of one sample; thread (tx, ty) adds partial rows ty, ty+32,
 // ... of column tx in ascending order, then one thread per column adds the 32
 // strands in ascending ty.  Every sum has one fixed association order, so the
@@ -98,7 +98,7 @@ __device__ __forceinline__ void store_scalar<bf16_t>(bf16_t *p, float v) {
 
 template <typename T>
 __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
-    T *__restrict__ out0, T *__restrict__ out1, const float *__restrict__ partial,
+    T *__restrict__ out0, T *__restrict__ out1, T *__restrict__ out2, const float *__restrict__ partial,
     int blocks_per_sample, int C, int ncols, int col_blocks) {
     __shared__ float strands[kRedStrands][kRedCols + 1];
     const int tx = threadIdx.x % kRedCols;
@@ -125,14 +125,12 @@ __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
         float s = strands[0][tx];
 #pragma unroll
         for (int i = 1; i < kRedStrands; ++i) s += strands[i][tx];
-        if (col < C)
-            store_scalar<T>(out0 + b * C + col, s);
-        else
-            store_scalar<T>(out1 + b * C + (col - C), s);
+        T *dst = col < C ? out0 : (col < 2 * C ? out1 : out2);  // column sets of C columns each
+        store_scalar<T>(dst + b * C + col % C, s);
     }
 }
 
-int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch,
+int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, int64_t batch,
                      int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
                      hipStream_t stream) {
     const int col_blocks = (int)((ncols + kRedCols - 1) / kRedCols);
@@ -140,10 +138,10 @@ int launch_colreduce(void *out0, void *out1, const float *partial, int64_t batch
     if (grid > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "column reducer grid too large");
     dim3 g((unsigned)grid), blk(kRedCols * kRedStrands);
     if (dtype == TT_NORM_BF16)
-        colreduce_kernel<bf16_t><<<g, blk, 0, stream>>>((bf16_t *)out0, (bf16_t *)out1, partial,
+        colreduce_kernel<bf16_t><<<g, blk, 0, stream>>>((bf16_t *)out0, (bf16_t *)out1, (bf16_t *)out2, partial,
                                                         blocks_per_sample, (int)C, (int)ncols, col_blocks);
     else
-        colreduce_kernel<float><<<g, blk, 0, stream>>>((float *)out0, (float *)out1, partial,
+        colreduce_kernel<float><<<g, blk, 0, stream>>>((float *)out0, (float *)out1, (float *)out2, partial,
                                                        blocks_per_sample, (int)C, (int)ncols, col_blocks);
     return check_launch("column reducer launch");
 }

@@ -327,7 +327,7 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
                               const float *rstd, const Map &map, int64_t rows, int dtype, void *ws,
                               size_t ws_bytes, hipStream_t stream) {
     // empty input: dweight is the empty sum, written by the reducer over zero partial rows
-    if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, 1, 0, C, C, dtype, stream);
+    if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, nullptr, 1, 0, C, C, dtype, stream);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
@@ -342,7 +342,7 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
     }
     st = check_launch("rmsnorm backward launch");
     if (st != TT_NORM_OK) return st;
-    return launch_colreduce(dw, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);
+    return launch_colreduce(dw, nullptr, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);
 }
 
 static int check_rms_args(const char *who, int64_t rows, int64_t cols, int dtype,

@@ -160,6 +160,68 @@ def modulated_layer_norm(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tens
     return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
 
 
+class GatedResidualAdaLNFunction(Function):
+    """(h2, out) = apply(h, attn, gate, scale, shift, epsilon):
+    h2 = h + attn * gate[:, None];  out = LayerNorm(h2) * (1 + scale[:, None]) + shift[:, None].
+
+    The residual update and the norm that follows it in the transformer blocks
+    (dit_layerspec.py:152-167, :351-352), which the reference runs as separate
+    elementwise kernels around the norm.  h, attn [B, S, C]; gate, scale, shift [B, C].
+    h2 is the new residual stream; its gradient from later uses is folded into the
+    same backward pass.  C must be 3072."""
+
+    @staticmethod
+    def forward(ctx, h, attn, gate, scale, shift, epsilon):
+        ext = _require_extension(fused_adaln, "fused_adaln")
+        _require_gpu(h, "GatedResidualAdaLNFunction")
+        cols = h.shape[-1]
+        if attn.shape != h.shape:
+            raise ValueError(f"attn {tuple(attn.shape)} must have the shape of h {tuple(h.shape)}")
+        mods = [t.contiguous().to(h.dtype) for t in (gate, scale, shift)]
+        if any(m.numel() != mods[0].numel() or m.numel() % cols for m in mods):
+            raise ValueError("gate, scale and shift must each hold [B, cols] elements")
+        batch = mods[0].numel() // cols
+        if batch > 1 and (h.dim() < 2 or h.shape[0] != batch):
+            raise ValueError(f"{batch} modulation rows need h.shape[0] == {batch}, got {tuple(h.shape)}")
+        h_c = _aligned_contiguous(h)
+        attn_c = _aligned_contiguous(attn.to(h.dtype))
+        rows = h_c.numel() // cols
+        h2 = torch.empty_like(h_c)
+        out = torch.empty_like(h_c)
+        mean = torch.empty(rows, device=h.device, dtype=torch.float32)
+        invvar = torch.empty(rows, device=h.device, dtype=torch.float32)
+        ext.torch_launch_gated_adaln_forward(h2, out, h_c, attn_c, mods[0], mods[1], mods[2], rows, cols,
+                                             float(epsilon), mean, invvar)
+        ctx.save_for_backward(h2, attn_c, mods[0], mods[1], mean, invvar)
+        ctx.rows, ctx.cols = rows, cols
+        ctx.mod_meta = [(t.shape, t.dtype) for t in (gate, scale, shift)]
+        ctx.attn_dtype = attn.dtype
+        ctx.set_materialize_grads(False)  # an unused h2 costs no zero tensor and no read
+        return h2, out
+
+    @staticmethod
+    def backward(ctx, grad_h2, grad_out):
+        h2, attn_c, gate_c, scale_c, mean, invvar = ctx.saved_tensors
+        if grad_out is None:
+            grad_out = torch.zeros_like(h2)
+        grad_out = _aligned_contiguous(grad_out.to(h2.dtype))
+        if grad_h2 is not None:
+            grad_h2 = _aligned_contiguous(grad_h2.to(h2.dtype))
+        dh = torch.empty_like(h2)
+        dattn = torch.empty_like(h2)
+        dgate, dscale, dshift = (torch.empty_like(scale_c) for _ in range(3))
+        fused_adaln.torch_launch_gated_adaln_backward(dh, dattn, dgate, dscale, dshift, grad_out, grad_h2, h2,
+                                                      attn_c, gate_c, scale_c, mean, invvar, ctx.rows, ctx.cols)
+        dgate, dscale, dshift = (g.reshape(shape).to(dtype)
+                                 for g, (shape, dtype) in zip((dgate, dscale, dshift), ctx.mod_meta))
+        return dh, dattn.to(ctx.attn_dtype), dgate, dscale, dshift, None
+
+
+def gated_residual_layer_norm(h, attn, gate, scale, shift, eps: float = 1e-6):
+    """Returns (h + attn * gate[:, None], modulated LayerNorm of that sum) from one fused pass."""
+    return GatedResidualAdaLNFunction.apply(h, attn, gate, scale, shift, eps)
+
+
 def _make_modulation_linear(embedding_dim: int, n_chunks: int, bias: bool, linear_parallel: bool, config):
     if not linear_parallel:
         return nn.Linear(embedding_dim, n_chunks * embedding_dim, bias=bias)

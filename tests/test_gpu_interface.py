@@ -159,6 +159,30 @@ def test_modulated_layer_norm_matches_unfused_norm2_site(FL, gpu_device):
     fwd_ok(got, want, O.adaln_excuse(d["x"], d["scale"], d["shift"], want))
 
 
+@pytest.mark.parametrize("use_h2", [True, False])
+def test_gated_residual_function_autograd(FL, gpu_device, use_h2):
+    """hidden = hidden + attn * gate.unsqueeze(1); norm2(hidden) * (1 + scale[:, None]) + shift[:, None]
+    (dit_layerspec.py:152-163) as one Function with two outputs; h2 either feeds a later use or not."""
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(2, 301, 3072, torch.bfloat16, seed=51, with_grad_h2=use_h2)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    leaves = [t.to(gpu_device).requires_grad_(True) for t in (h, a, q, sc, sh)]
+    h2, out = FL.gated_residual_layer_norm(*leaves, eps=EPS)
+    assert torch.equal(h2.detach().cpu(), want[0])
+    fwd_ok(out, want[1], O.adaln_excuse(want[0], sc, sh, want[1]))
+    if use_h2:
+        torch.autograd.backward([out, h2], [go.to(gpu_device), g2.to(gpu_device)])
+    else:
+        out.backward(go.to(gpu_device))
+    terms = want[2].float().abs() + (g2.float().abs() if use_h2 else 0)
+    assert O.frac_outside(leaves[0].grad.cpu(), want[2], 1e-2, 1e-3, magnitude=terms) <= 1e-5
+    assert O.frac_outside(leaves[1].grad.cpu(), want[3], 1e-2, 1e-3,
+                          magnitude=terms * q.float().abs()[:, None]) <= 1e-5
+    assert leaves[2].grad.shape == q.shape and leaves[2].grad.dtype == q.dtype
+    assert O.colsum_outside(leaves[2].grad.cpu(), want[4], terms * a.float(), dim=1) == 0
+    grad_ok(leaves[3].grad, want[5])
+    grad_ok(leaves[4].grad, want[6])
+
+
 def test_reference_signature_extension_calls(FL, gpu_device):
     """Drive the extension exactly as the reference's autograd classes do
     (dit_fusedlayers.py:95-104,128-136,305-313,337-346)."""

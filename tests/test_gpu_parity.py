@@ -246,6 +246,105 @@ def test_full_size_adaln_properties(capi, gpu_device):
     assert_grad_bf16(dx[:, idx], want_dx, "dx rows", allow=1e-5)
 
 
+# ---------------------------------------------------- gated residual + AdaLN
+
+def _gated_terms(want_dh, grad_h2):
+    t = want_dh.float().abs()
+    return t if grad_h2 is None else t + grad_h2.float().abs()
+
+
+@pytest.mark.parametrize("batch,seq,with_h2_grad", [(1, 1, True), (1, 7, False), (2, 1031, True),
+                                                     (3, 333, False), (5, 1001, True), (260, 3, True)])
+def test_gated_residual_adaln_bf16_vs_eager(capi, gpu_device, batch, seq, with_h2_grad):
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(batch, seq, 3072, torch.bfloat16, seed=300 + seq % 83,
+                                                  with_grad_h2=with_h2_grad)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    w_h2, w_out, w_dh, w_da, w_dq, w_dsc, w_dsh = want
+    to = lambda t: None if t is None else t.to(gpu_device)
+    H, A, Q, SC, SH, GO, G2 = (to(t) for t in (h, a, q, sc, sh, go, g2))
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(H, A, Q, SC, SH, EPS)
+    assert torch.equal(h2.cpu(), w_h2)                      # two roundings, both fixed by the expression
+    assert_fwd_bf16(out, w_out, O.adaln_excuse(w_h2, sc, sh, w_out), "out")
+    _, want_mu, want_r = O.staged_adaln_fwd(w_h2, sc, sh)
+    torch.testing.assert_close(rstd.cpu(), want_r.reshape(-1), rtol=2e-6, atol=0)
+    torch.testing.assert_close(mean.cpu(), want_mu.reshape(-1), rtol=0, atol=2e-6)
+    dh, da, dq, dsc, dsh = capi.gated_residual_adaln_backward(GO, G2, h2, A, Q, SC, mean, rstd)
+    # gradients: |got - want| <= 1e-3 + 1e-2 * m on all but 1e-5 of elements; m = |want| except for
+    # dh = round(dx of the norm) + grad_h2, a sum of separately rounded terms that may cancel, where
+    # m is the size of the terms; dgate sums dh * attn with dh known to an ulp: random-walk bound
+    terms = _gated_terms(w_dh, g2)
+    assert O.frac_outside(dh.cpu(), w_dh, 1e-2, 1e-3, magnitude=terms) <= 1e-5
+    assert O.frac_outside(da.cpu(), w_da, 1e-2, 1e-3, magnitude=terms * q.float().abs()[:, None]) <= 1e-5
+    assert O.colsum_outside(dq.cpu(), w_dq, terms * a.float(), dim=1) == 0
+    assert_grad_bf16(dsc, w_dsc, "dscale")
+    assert_grad_bf16(dsh, w_dsh, "dshift")
+
+
+def test_gated_residual_adaln_fp32_vs_eager(capi, gpu_device):
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(3, 171, 3072, torch.float32, seed=12)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    H, A, Q, SC, SH, GO, G2 = (t.to(gpu_device) for t in (h, a, q, sc, sh, go, g2))
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(H, A, Q, SC, SH, EPS)
+    dh, da, dq, dsc, dsh = capi.gated_residual_adaln_backward(GO, G2, h2, A, Q, SC, mean, rstd)
+    torch.testing.assert_close(h2.cpu(), want[0], rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(out.cpu(), want[1], rtol=1e-5, atol=1e-6)   # forward fp32: rel 1e-5
+    for got, w in zip((dh, da), want[2:4]):                                # gradients fp32: rel 1e-4
+        torch.testing.assert_close(got.cpu(), w, rtol=1e-4, atol=1e-5)
+    l1 = (want[2].abs() * a.abs()).sum(1)
+    assert ((dq.cpu() - want[4]).abs() <= 1e-4 * l1 + 1e-5).all()          # column sums: 1e-4 of the L1 mass
+    for got, w in zip((dsc, dsh), want[5:7]):
+        torch.testing.assert_close(got.cpu(), w, rtol=1e-4, atol=1e-4)
+
+
+def test_full_size_gated_residual_adaln_properties(capi, gpu_device):
+    """118 800 x 3072 bf16.  The fused op must be bit-identical to its parts run one after the
+    other: h2 to the elementwise update, out / mean / rstd to the plain AdaLN forward of h2, and the
+    backward to the plain AdaLN backward followed by the elementwise gradient formulas."""
+    rows, C = _full_rows(), 3072
+    gen = torch.Generator(device=gpu_device).manual_seed(2)
+    rnd = lambda *shape, s=1.0: (s * torch.randn(*shape, device=gpu_device, generator=gen)).bfloat16()
+    h, a, go = rnd(1, rows, C), rnd(1, rows, C), rnd(1, rows, C, s=0.1)
+    q, sc, sh = rnd(1, C, s=0.3), rnd(1, C, s=0.3), rnd(1, C, s=0.3)
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(h, a, q, sc, sh, EPS)
+    assert torch.equal(h2, h + a * q[:, None])
+    out_p, mean_p, rstd_p = capi.adaln_forward(h2, sc, sh, EPS)
+    assert torch.equal(out, out_p) and torch.equal(mean, mean_p) and torch.equal(rstd, rstd_p)
+    del out_p, h
+    dh, da, dq, dsc, dsh = capi.gated_residual_adaln_backward(go, None, h2, a, q, sc, mean, rstd)
+    dx_p, dsc_p, dsh_p = capi.adaln_backward(go, h2, sc, mean, rstd)
+    assert torch.equal(dh, dx_p) and torch.equal(dsc, dsc_p) and torch.equal(dsh, dsh_p)
+    del dx_p
+    assert torch.equal(da, dh * q[:, None])
+    want_dq = (dh * a).float().sum(1)
+    assert O.colsum_outside(dq.cpu(), want_dq.cpu(), (dh * a).float().cpu(), dim=1, ulp=2.0 ** -9) == 0
+    del da
+    # with an upstream gradient on h2: dh = round(dx of the norm + that gradient), run twice -> identical
+    g2 = rnd(1, rows, C, s=0.1)
+    dh2a = capi.gated_residual_adaln_backward(go, g2, h2, a, q, sc, mean, rstd)
+    assert torch.equal(dh2a[0], dh + g2)
+    dh2b = capi.gated_residual_adaln_backward(go, g2, h2, a, q, sc, mean, rstd)
+    assert all(torch.equal(x, y) for x, y in zip(dh2a, dh2b))
+    # gate = 0: the residual stream passes through, attn receives no gradient
+    z = torch.zeros_like(q)
+    h2z, _, mz, rz = capi.gated_residual_adaln_forward(h2, a, z, sc, sh, EPS)
+    assert torch.equal(h2z, h2)
+    daz = capi.gated_residual_adaln_backward(go, None, h2z, a, z, sc, mz, rz)[1]
+    assert not daz.any()
+
+
+def test_gated_residual_adaln_rejects_other_widths(capi, gpu_device):
+    mk = lambda *shape: torch.zeros(*shape, device=gpu_device, dtype=torch.bfloat16)
+    with pytest.raises(capi.NormError) as e:
+        capi.gated_residual_adaln_forward(mk(1, 8, 128), mk(1, 8, 128), mk(1, 128), mk(1, 128), mk(1, 128), EPS)
+    assert e.value.status == 2
+    # zero rows: a no-op forward and all-zero parameter gradients
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(mk(2, 0, 3072), mk(2, 0, 3072), mk(2, 3072),
+                                                            mk(2, 3072), mk(2, 3072), EPS)
+    grads = capi.gated_residual_adaln_backward(mk(2, 0, 3072), None, h2, mk(2, 0, 3072), mk(2, 3072),
+                                               mk(2, 3072), mean, rstd)
+    assert all(g.shape == (2, 3072) and not g.any() for g in grads[2:])
+
+
 def test_qk_norm_shape_one_cp_rank(capi, gpu_device):
     """q of one CP=4 rank: [1, 29700, 24, 128] bf16 = 712 800 rows of 128."""
     d = O.make_rmsnorm_inputs((1, 29700, 24), 128, torch.bfloat16, seed=0)

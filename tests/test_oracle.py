@@ -262,6 +262,91 @@ def test_adaln_c_f32_matches_eager():
 
 # ------------------------------------------------------------ golden vectors
 
+# ----------------------------------------------------- gated residual + AdaLN
+
+def test_gated_bruteforce_loops_fp64():
+    """Scalar loops over a tiny case: catches gate applied to h instead of attn, gate of the wrong
+    sample, the norm taken of h instead of h2, a gradient of h2 that misses either of its two uses."""
+    gen = torch.Generator().manual_seed(31)
+    B, S, C = 2, 3, 8
+    h, a, go, g2 = (torch.randn(B, S, C, generator=gen, dtype=torch.float64) for _ in range(4))
+    q, sc, sh = (0.5 * torch.randn(B, C, generator=gen, dtype=torch.float64) for _ in range(3))
+    h2, out, dh, da, dq, dsc, dsh = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2, EPS)
+    for b in range(B):
+        dq_want = [0.0] * C
+        for s in range(S):
+            row = [float(h[b, s, c]) + float(a[b, s, c]) * float(q[b, c]) for c in range(C)]
+            mu = sum(row) / C
+            var = sum((v - mu) ** 2 for v in row) / C
+            r = 1.0 / math.sqrt(var + EPS)
+            xhat = [(v - mu) * r for v in row]
+            gx = [float(go[b, s, c]) * (1.0 + float(sc[b, c])) for c in range(C)]
+            m1 = sum(gx) / C
+            m2 = sum(gx[c] * xhat[c] for c in range(C)) / C
+            for c in range(C):
+                assert abs(float(h2[b, s, c]) - row[c]) < 1e-12
+                want = xhat[c] * (1.0 + float(sc[b, c])) + float(sh[b, c])
+                assert abs(float(out[b, s, c]) - want) < 1e-9
+                dh_want = r * (gx[c] - m1 - xhat[c] * m2) + float(g2[b, s, c])
+                assert abs(float(dh[b, s, c]) - dh_want) < 1e-9
+                assert abs(float(da[b, s, c]) - dh_want * float(q[b, c])) < 1e-9
+                dq_want[c] += dh_want * float(a[b, s, c])
+        for c in range(C):
+            assert abs(float(dq[b, c]) - dq_want[c]) < 1e-9
+    # the float64 closed form agrees with autograd on every output
+    truth = O.truth_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2, EPS)
+    for got, want in zip((h2, out, dh, da, dq, dsc, dsh), truth):
+        torch.testing.assert_close(got, want, rtol=1e-9, atol=1e-11)
+    # without a gradient at h2, dh is the norm's dx alone
+    no2 = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, None, EPS)
+    torch.testing.assert_close(no2[2] + g2, dh, rtol=1e-9, atol=1e-11)
+
+
+def test_gated_gradcheck_and_special_cases():
+    gen = torch.Generator().manual_seed(32)
+    B, S, C = 2, 2, 12
+    mk = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    leaves = [mk(B, S, C), mk(B, S, C), 0.3 * mk(B, C), 0.3 * mk(B, C), 0.3 * mk(B, C)]
+    for t in leaves:
+        t.requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda *a: O.eager_gated_residual_adaln(*a, EPS), leaves, eps=1e-6, atol=1e-6)
+    h, a, q, sc, sh = (t.detach() for t in leaves)
+    # gate = 0: the residual stream passes through untouched and the op is the plain modulated norm
+    h2, out = O.eager_gated_residual_adaln(h, a, torch.zeros_like(q), sc, sh, EPS)
+    assert torch.equal(h2, h)
+    torch.testing.assert_close(out, O.eager_adaln(h, sc, sh, EPS), rtol=0, atol=0)
+    # gate = 1, attn = -h: h2 = 0, every row is constant, the norm returns shift
+    h2, out = O.eager_gated_residual_adaln(h, -h, torch.ones_like(q), sc, sh, EPS)
+    assert h2.abs().max() == 0
+    torch.testing.assert_close(out, sh[:, None].expand_as(out), rtol=0, atol=1e-12)
+
+
+def test_gated_staged_agrees_with_eager_bf16():
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(2, 48, 3072, torch.bfloat16, seed=33)
+    eh2, eout, edh, eda, edq, edsc, edsh = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    sh2, sout, smu, sr = O.staged_gated_residual_adaln_fwd(h, a, q, sc, sh)
+    assert torch.equal(sh2, eh2)  # two roundings, both fixed by the eager expression
+    rep = O.compare_bf16_ulp(sout, eout, excuse_abs=O.adaln_excuse(eh2, sc, sh, eout))
+    assert rep.n_gt1 == 0 and rep.n_excused < 1e-4 * rep.n and rep.frac_exact > 0.999, rep
+    # dropping the rounding of attn*gate is visible in h2
+    single = (h.float() + a.float() * q.float()[:, None]).bfloat16()
+    assert (single != eh2).float().mean() > 0.02
+    sdh, sda, sdq, sdsc, sdsh = O.staged_gated_residual_adaln_bwd(eh2, a, q, sc, smu, sr, go, g2)
+    # dh sums two rounded terms: a one-ulp disagreement in the norm's dx survives a cancelling sum,
+    # so its bound scales with the terms (|dh| + |grad_h2| >= |dx of the norm|)
+    terms = edh.float().abs() + g2.float().abs()
+    assert O.frac_outside(sdh, edh, 1e-2, 1e-3, magnitude=terms) < 1e-5
+    assert O.frac_outside(sda, eda, 1e-2, 1e-3, magnitude=terms * q.float().abs()[:, None]) < 1e-5
+    for got, want in ((sdsc, edsc), (sdsh, edsh)):
+        assert O.frac_outside(got, want, 1e-2, 1e-3) == 0.0
+    # dgate sums dh*attn, and dh is known to an ulp only: random-walk bound on the column
+    assert O.colsum_outside(sdq, edq, terms * a.float(), dim=1) == 0
+    # and the float64 truth is within bf16 rounding noise of both
+    truth = O.truth_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    assert O.frac_outside(sdh, truth[2], 2e-2, 2e-2) < 1e-4
+    assert O.colsum_outside(sdq, truth[4], terms * a.float(), dim=1) == 0
+
+
 def test_golden_vectors_reproduce():
     gold = load_golden()
     assert len(gold) == 7
