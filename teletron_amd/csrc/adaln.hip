@@ -22,6 +22,9 @@
 #ifndef TTN_ADALN_BWD_ROW_BUFFERS
 #define TTN_ADALN_BWD_ROW_BUFFERS 1
 #endif
+#ifndef TTN_GATED_LATE_OPERANDS  // gated backward, 2-byte rows: fetch attn and e in the second pass
+#define TTN_GATED_LATE_OPERANDS 0
+#endif
 #ifndef TTN_ADALN_BWD_PREFETCH_MID
 #define TTN_ADALN_BWD_PREFETCH_MID 0
 #endif
@@ -239,6 +242,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     // gate[sample]: unpacked once for 2-byte elements; 4-byte rows have no registers to spare and
     // re-read it (cache hits) where it is used
     constexpr bool kGateResident = GATED && sizeof(T) == 2;
+    constexpr bool kEarlyOperands = kGateResident && !TTN_GATED_LATE_OPERANDS;  // attn, e fetched with g, x
     [[maybe_unused]] float gatev[kGateResident ? CHUNKS : 1][VEC];
     if constexpr (kGateResident) {
 #pragma unroll
@@ -256,7 +260,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 
     struct RowRegs {
         u32x4 g[CHUNKS], x[CHUNKS];
-        u32x4 a[kGateResident ? CHUNKS : 1], e[kGateResident ? CHUNKS : 1];
+        u32x4 a[kEarlyOperands ? CHUNKS : 1], e[kEarlyOperands ? CHUNKS : 1];
         float r, mu;
         int64_t row;
         bool ok;
@@ -279,7 +283,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
 #endif
-        if constexpr (kGateResident) {  // 4-byte rows fetch these two where they are used instead
+        if constexpr (kEarlyOperands) {  // otherwise these two are fetched where they are used
             const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + b.row * C) + l;
             const u32x4 *pe = reinterpret_cast<const u32x4 *>(e + b.row * C) + l;
 #pragma unroll
@@ -348,7 +352,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             if constexpr (GATED) {
                 float ev[VEC], av[VEC], dav[VEC];
                 E::round(o);  // the norm's dx, materialised in the element type
-                if constexpr (kGateResident) {
+                if constexpr (kEarlyOperands) {
                     E::unpack(b.e[k], ev);
                     E::unpack(b.a[k], av);
                 } else {
