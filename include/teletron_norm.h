@@ -1,6 +1,10 @@
 /* teletron_norm.h -- C ABI of the gfx950 fused normalization library
  * (libteletron_norm.so): fused RMSNorm and fused AdaLayerNorm, forward and
- * backward, for bf16 and fp32 rows of 128 or 3072 columns.
+ * backward.  Tuned kernels for bf16 and fp32 rows of 128 or 3072 columns (the
+ * shapes the reference's kernels are built for, teletron/models/dit/
+ * dit_fusedlayers.py:91,301); any-width kernels for every other row of whole
+ * 16-byte pieces, bf16 / fp16 / fp32, up to 8192 two-byte or 4096 four-byte
+ * columns, behind the same native entry points.
  *
  * This is the seam the reference has between its pybind glue and its kernel
  * launchers (teletron_op/fused_rmsnorm/include/rmsnorm_kernel.h:5-25 and
@@ -42,7 +46,7 @@ extern "C" {
 enum tt_norm_status {
     TT_NORM_OK = 0,
     TT_NORM_EINVAL = 1,       /* null pointer, negative size, non-positive cols or batch */
-    TT_NORM_EUNSUPPORTED = 2, /* cols or dtype the kernels are not built for */
+    TT_NORM_EUNSUPPORTED = 2, /* cols or dtype this entry point is not built for */
     TT_NORM_EALIGN = 3,       /* a tensor pointer is not 16-byte aligned */
     TT_NORM_EWORKSPACE = 4,   /* workspace missing or smaller than *_workspace_bytes() */
     TT_NORM_EHIP = 5          /* the HIP runtime refused the launch; see tt_norm_last_error() */
@@ -50,7 +54,8 @@ enum tt_norm_status {
 
 enum tt_norm_dtype {
     TT_NORM_BF16 = 0,
-    TT_NORM_F32 = 1
+    TT_NORM_F32 = 1,
+    TT_NORM_F16 = 2 /* any-width kernels only */
 };
 
 /* ABI version of the loaded library (TT_NORM_ABI_VERSION at build time). */
@@ -62,8 +67,14 @@ const char *tt_norm_status_string(int status);
 /* Thread-local detail of the last non-OK status returned on this thread. */
 const char *tt_norm_last_error(void);
 
-/* 1 if (cols, dtype) is a shape the kernels are built for, else 0. */
+/* 1 if the native entry points (tt_rmsnorm_forward/backward, tt_adaln_forward/backward and
+ * their workspace queries) accept (cols, dtype), else 0. */
 int tt_norm_supported(int64_t cols, int dtype);
+
+/* 1 if (cols, dtype) is one of the tuned shapes (cols 128 or 3072, bf16 or fp32): the only
+ * ones the reference-contract (*_from_out, *_xnorm, *_from_xnorm) and strided entry points
+ * take; the gated residual entry points take cols 3072 only. */
+int tt_norm_tuned(int64_t cols, int dtype);
 
 /* ------------------------------------------------------------------ RMSNorm
  * out = round(round(x * rstd) * weight),  rstd = 1/sqrt(mean_c(x^2) + eps)

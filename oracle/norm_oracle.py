@@ -229,7 +229,7 @@ def truth_adaln_fwd_bwd(x, scale, shift, grad, eps: float = EPS):
 def bf16_ordinal(t: torch.Tensor) -> torch.Tensor:
     """Monotone integer index of each bf16 value (adjacent values differ by 1;
     +0 and -0 share index 0)."""
-    assert t.dtype == torch.bfloat16
+    assert t.dtype in (torch.bfloat16, torch.float16)  # both are 16-bit sign-magnitude patterns
     bits = t.contiguous().view(torch.int16).to(torch.int32)
     return torch.where(bits >= 0, bits, -(bits & 0x7FFF))
 
@@ -280,19 +280,25 @@ def compare_bf16_ulp(got: torch.Tensor, want: torch.Tensor,
                      max_ulp=int(d.max()) if d.numel() else 0)
 
 
+def _ulp_rel(dtype: torch.dtype) -> float:
+    """Largest relative size of one ulp: 2^-7 for bf16 (8 significant bits), 2^-10 for fp16 (11)."""
+    return 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+
+
 def rmsnorm_excuse(want_out: torch.Tensor) -> torch.Tensor:
-    """out = rnd(y*w): one-ulp step of y (<= 2^-7 |y*w|) plus one ulp of out."""
-    return want_out.float().abs() * 2.0 ** -6
+    """out = rnd(y*w): one-ulp step of y (<= u |y*w|) plus one ulp of out; u = 2^-7 for bf16."""
+    return want_out.float().abs() * (2 * _ulp_rel(want_out.dtype))
 
 
 def adaln_excuse(x, scale, shift, want_out, eps: float = EPS) -> torch.Tensor:
     """out = rnd(rnd(xn*t) + shift): one-ulp step of xn carried through t
-    (<= 2^-7 |p|), one ulp of p (<= 2^-7 |p|), one ulp of out (<= 2^-7 |out|)."""
+    (<= u |p|), one ulp of p (<= u |p|), one ulp of out (<= u |out|); u = 2^-7 for bf16."""
     B, C = scale.shape
     x3 = x.reshape(B, -1, C)
     xn = F.layer_norm(x3, (C,), None, None, eps)
     p = (xn * (1 + scale[:, None])).float().abs().reshape(want_out.shape)
-    return p * 2.0 ** -6 + want_out.float().abs() * 2.0 ** -7
+    u = _ulp_rel(want_out.dtype)
+    return p * (2 * u) + want_out.float().abs() * u
 
 
 def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float,
@@ -306,6 +312,19 @@ def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float
         return 0.0
     m = w.abs() if magnitude is None else magnitude.double().cpu().abs()
     return float(((g - w).abs() > atol + rtol * m).double().mean())
+
+
+def adaln_dx_terms(x, scale, grad, eps: float = EPS) -> torch.Tensor:
+    """Size of the three terms LayerNorm's backward adds, r*(|gx| + |mean gx| + |xhat * mean(gx*xhat)|).
+    For short rows the two means are not small and the terms cancel; eager on the CPU moreover keeps
+    mean and rstd of a 16-bit input in 16 bits, so its dx carries that rounding times the terms.
+    Used as `magnitude` of frac_outside for dx of narrow rows."""
+    xf = x.float()
+    mu = xf.mean(-1, keepdim=True)
+    r = torch.rsqrt(((xf - mu) ** 2).mean(-1, keepdim=True) + eps)
+    xhat = (xf - mu) * r
+    gx = (grad * (1 + scale[:, None])).float()
+    return r * (gx.abs() + gx.mean(-1, keepdim=True).abs() + (xhat * (gx * xhat).mean(-1, keepdim=True)).abs())
 
 
 def colsum_outside(got: torch.Tensor, want: torch.Tensor, terms: torch.Tensor, dim: int,

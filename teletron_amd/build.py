@@ -23,10 +23,13 @@ LIB_PATH = os.path.join(LIB_DIR, "libteletron_norm.so")
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 ARCH = "gfx950"
-# -packed-fp32-ops off: scalar fp32 VALU only (packed fp32 forms are not trusted on this fleet)
+# -packed-fp32-ops off: scalar fp32 VALU only (packed fp32 forms are not trusted on this fleet).
+# -ffp-contract=off: the kernels reproduce the eager graph's rounding points, so a multiply and a
+# later add must stay two roundings unless the source says fmaf; with contraction allowed the
+# compiler narrows fp16 chains to half arithmetic and then fuses across a rounding point.
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip"]
+             "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip"]
 EXT_MODULES = {"fused_rmsnorm": "fused_rmsnorm_ext.cpp", "fused_adaln": "fused_adaln_ext.cpp"}
 
 
@@ -40,11 +43,18 @@ def _run(cmd, cwd=None):
 
 
 def build_kernels(verbose: bool = True) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [HIPCC, *HIP_FLAGS, "-shared", "-o", LIB_PATH] + KERNEL_SOURCES
-    out = _run(cmd, cwd=CSRC)
+    """Each source is compiled to an object of its own (in parallel), then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    objs = [os.path.join(obj_dir, os.path.splitext(src)[0] + ".o") for src in KERNEL_SOURCES]
+    with ThreadPoolExecutor(max_workers=min(4, len(KERNEL_SOURCES))) as pool:
+        logs = list(pool.map(lambda so: _run([HIPCC, *HIP_FLAGS, "-c", so[0], "-o", so[1]], cwd=CSRC),
+                             zip(KERNEL_SOURCES, objs)))
+    logs.append(_run([HIPCC, "--offload-arch=" + ARCH, "-fPIC", "-shared", "-o", LIB_PATH] + objs))
     if verbose:
-        print("built", os.path.relpath(LIB_PATH, ROOT), out.strip())
+        print("built", os.path.relpath(LIB_PATH, ROOT), "\n".join(l for l in logs if l.strip()).strip())
     return LIB_PATH
 
 

@@ -14,11 +14,11 @@ import torch
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libteletron_norm.so")
 
-BF16, F32 = 0, 1
-_DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
+BF16, F32, F16 = 0, 1, 2
+_DTYPES = {torch.bfloat16: BF16, torch.float32: F32, torch.float16: F16}
 
 EXPORTS = (
-    "tt_norm_abi_version", "tt_norm_status_string", "tt_norm_last_error", "tt_norm_supported",
+    "tt_norm_abi_version", "tt_norm_status_string", "tt_norm_last_error", "tt_norm_supported", "tt_norm_tuned",
     "tt_rmsnorm_forward", "tt_rmsnorm_backward_workspace_bytes", "tt_rmsnorm_backward",
     "tt_rmsnorm_backward_from_out", "tt_rmsnorm_forward_strided", "tt_rmsnorm_backward_strided",
     "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
@@ -50,6 +50,7 @@ def lib() -> ctypes.CDLL:
         L.tt_norm_status_string.argtypes = [ci]
         L.tt_norm_last_error.restype = ctypes.c_char_p
         L.tt_norm_supported.argtypes = [i64, ci]
+        L.tt_norm_tuned.argtypes = [i64, ci]
         L.tt_rmsnorm_forward.argtypes = [vp, vp, vp, vp, i64, i64, dbl, ci, vp]
         L.tt_rmsnorm_backward_workspace_bytes.restype = sz
         L.tt_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64, ci]

@@ -483,14 +483,19 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
                             NSETS * C, dtype, a.stream);
 }
 
+// tuned_only: the entry point exists for the tuned shapes only (reference-contract and gated forms).
 static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sample, int64_t cols,
-                            int dtype, std::initializer_list<const void *> ptrs) {
+                            int dtype, std::initializer_list<const void *> ptrs, bool tuned_only = false) {
     if (batch <= 0 || rows_per_sample < 0 || cols <= 0)
         return fail(TT_NORM_EINVAL, "%s: batch=%lld rows_per_sample=%lld cols=%lld", who, (long long)batch,
                     (long long)rows_per_sample, (long long)cols);
-    if (!tt_norm_supported(cols, dtype))
-        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
+    if (tuned_only && !tuned_shape(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072, bf16/fp32)", who,
                     (long long)cols, dtype);
+    if (!tt_norm_supported(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED,
+                    "%s: cols=%lld dtype=%d (cols must be a multiple of 16 bytes of elements, at most 8192 "
+                    "two-byte or 4096 four-byte; dtype bf16, fp16 or fp32)", who, (long long)cols, dtype);
     if (rows_per_sample == 0) return TT_NORM_OK;  // empty input: nothing is dereferenced
     for (const void *p : ptrs) {
         if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
@@ -522,6 +527,9 @@ int tt_adaln_forward(void *out, float *mean, float *rstd, const void *x, const v
     int st = check_adaln_args("tt_adaln_forward", batch, rows_per_sample, cols, dtype, {out, x, scale, shift});
     if (st != TT_NORM_OK) return st;
     if ((!mean || !rstd) && rows_per_sample > 0) return fail(TT_NORM_EINVAL, "tt_adaln_forward: null mean/rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_adaln_forward(out, mean, rstd, x, scale, shift, batch, rows_per_sample, cols, eps, dtype,
+                                      (hipStream_t)stream);
     const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
 #define CALL(T, C) return adaln_forward_t<T, C, false>(out, nullptr, mean, rstd, x, scale, shift, a)
     TTN_DISPATCH(dtype, cols, CALL);
@@ -532,7 +540,7 @@ int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x, 
                            const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols,
                            double eps, int dtype, void *stream) {
     int st = check_adaln_args("tt_adaln_forward_xnorm", batch, rows_per_sample, cols, dtype,
-                              {out, x_norm, x, scale, shift});
+                              {out, x_norm, x, scale, shift}, true);
     if (st != TT_NORM_OK) return st;
     if (!rstd && rows_per_sample > 0) return fail(TT_NORM_EINVAL, "tt_adaln_forward_xnorm: null rstd");
     const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
@@ -543,6 +551,7 @@ int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x, 
 
 size_t tt_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
     if (batch <= 0 || rows_per_sample <= 0 || !tt_norm_supported(cols, dtype)) return 0;
+    if (!tuned_shape(cols, dtype)) return anywidth_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return 0;
@@ -560,6 +569,9 @@ int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, co
     if (st != TT_NORM_OK) return st;
     if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward: null dscale/dshift/mean/rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols,
+                                       dtype, workspace, workspace_bytes, (hipStream_t)stream);
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
 #define CALL(T, C)                                                                                \
     return adaln_backward_t<T, C, false>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype, workspace, \
@@ -573,7 +585,7 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                  int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                  void *workspace, size_t workspace_bytes, void *stream) {
     int st = check_adaln_args("tt_adaln_backward_from_xnorm", batch, rows_per_sample, cols, dtype,
-                              {dx, dout, x_norm, scale});
+                              {dx, dout, x_norm, scale}, true);
     if (st != TT_NORM_OK) return st;
     if (!dscale || !dshift || (!rstd && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward_from_xnorm: null dscale/dshift/rstd");
@@ -592,7 +604,7 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
                                     const void *shift, int64_t batch, int64_t rows_per_sample,
                                     int64_t cols, double eps, int dtype, void *stream) {
     int st = check_adaln_args("tt_gated_residual_adaln_forward", batch, rows_per_sample, cols, dtype,
-                              {h2, out, h, attn, gate, scale, shift});
+                              {h2, out, h, attn, gate, scale, shift}, true);
     if (st != TT_NORM_OK) return st;
     if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_forward: built for cols 3072 only");
     if ((!mean || !rstd) && rows_per_sample > 0)
@@ -617,7 +629,7 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                      int64_t cols, int dtype, void *workspace, size_t workspace_bytes,
                                      void *stream) {
     int st = check_adaln_args("tt_gated_residual_adaln_backward", batch, rows_per_sample, cols, dtype,
-                              {dh, dattn, dout, h2, attn, gate, scale});
+                              {dh, dattn, dout, h2, attn, gate, scale}, true);
     if (st != TT_NORM_OK) return st;
     if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_backward: built for cols 3072 only");
     if (dh2 && !aligned16(dh2)) return fail(TT_NORM_EALIGN, "tt_gated_residual_adaln_backward: dh2 not 16-byte aligned");

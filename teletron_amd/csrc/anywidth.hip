@@ -1,0 +1,650 @@
+// RMSNorm and AdaLN for any row width: cols a multiple of one 16-byte access
+// (8 two-byte or 4 four-byte elements), up to 1024 accesses per row (8192 / 4096
+// columns), for bf16, fp16 and fp32.  The widths and types the tuned kernels in
+// rmsnorm.hip / adaln.hip are not built for land here, so that smaller models
+// (other hidden sizes and head dimensions) still run fused.
+//
+// Same arithmetic and rounding points as the tuned kernels, same row -> lane
+// geometry, but the width is a run-time argument: a row is laid over a padded
+// geometry of LANES x CHUNKS accesses (the smallest instantiated one that holds
+// it) and every lane knows which of its accesses fall inside the row.  Accesses
+// outside read zeros and write nothing.  The parameter-gradient reduction is
+// the same fixed-order two-stage scheme, so results are bit-identical from run
+// to run.
+#include <hip/hip_runtime.h>
+
+#include "norm_device.h"
+#include "norm_host.h"
+
+namespace ttn {
+
+template <typename T, int LANES_, int CHUNKS_>
+struct PadGeom {
+    static constexpr int VEC = Elem<T>::VEC;
+    static constexpr int LANES = LANES_;
+    static constexpr int CHUNKS = CHUNKS_;
+    static constexpr int RPW = kWaveSize / LANES;
+    static_assert(LANES == 16 || LANES == 32 || LANES == 64, "row must fill whole DPP rows");
+    static_assert(LANES == 64 || CHUNKS == 1, "only full wavefronts take several accesses per lane");
+};
+
+// Which of this lane's accesses lie inside a row of `pieces` 16-byte pieces.
+template <typename G>
+struct LaneMask {
+    bool in[G::CHUNKS];
+    __device__ __forceinline__ LaneMask(int l, int pieces) {
+#pragma unroll
+        for (int k = 0; k < G::CHUNKS; ++k) in[k] = k * G::LANES + l < pieces;
+    }
+};
+
+template <typename G>
+__device__ __forceinline__ void load_row(u32x4 (&dst)[G::CHUNKS], const void *row_base, int l, bool ok,
+                                         const LaneMask<G> &m) {
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(row_base) + l;
+#pragma unroll
+    for (int k = 0; k < G::CHUNKS; ++k) dst[k] = (ok && m.in[k]) ? load16_stream(p + k * G::LANES) : u32x4{0, 0, 0, 0};
+}
+
+template <typename G>
+__device__ __forceinline__ void load_param(u32x4 (&dst)[G::CHUNKS], const void *base, int l, const LaneMask<G> &m) {
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(base) + l;
+#pragma unroll
+    for (int k = 0; k < G::CHUNKS; ++k) dst[k] = m.in[k] ? load16(p + k * G::LANES) : u32x4{0, 0, 0, 0};
+}
+
+// Workgroup-level flush of per-lane column sums: rows of a wavefront folded by
+// shuffles, wavefronts added into LDS in wavefront order, one fp32 row of
+// NSETS*C partial sums written out.  lds holds NSETS*C floats.
+template <typename G, int NSETS>
+__device__ __forceinline__ void flush_partials_anywidth(float (&acc)[NSETS][G::CHUNKS][G::VEC],
+                                                        float *__restrict__ partial_row, float *lds, int C,
+                                                        const LaneMask<G> &m) {
+    constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s)
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[s][k][j] = fold_rows_of_wave<LANES>(acc[s][k][j]);
+    for (int wv = 0; wv < kRowWaves; ++wv) {
+        if (wave == wv && sub == 0) {
+#pragma unroll
+            for (int s = 0; s < NSETS; ++s)
+#pragma unroll
+                for (int k = 0; k < CHUNKS; ++k) {
+                    if (!m.in[k]) continue;
+                    float *p = lds + s * C + (k * LANES + l) * VEC;
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) p[j] = (wv == 0) ? acc[s][k][j] : p[j] + acc[s][k][j];
+                }
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < NSETS * C; i += kRowThreads) partial_row[i] = lds[i];
+}
+
+// ------------------------------------------------------------------ RMSNorm
+
+template <typename T, int LANES, int CHUNKS>
+__global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
+    T *__restrict__ out, float *__restrict__ rstd, const T *__restrict__ x, const T *__restrict__ w,
+    int64_t rows, int C, float eps) {
+    using G = PadGeom<T, LANES, CHUNKS>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, RPW = G::RPW;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const LaneMask<G> m(l, C / VEC);
+
+    u32x4 wr[CHUNKS];
+    load_param<G>(wr, w, l, m);
+
+    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(wr);
+        const int64_t row = grp * RPW + sub;
+        const bool ok = row < rows;
+        u32x4 xr[CHUNKS];
+        load_row<G>(xr, x + row * C, l, ok, m);
+
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) ss = fmaf(v[j], v[j], ss);
+        }
+        ss = group_sum<LANES>(ss);
+        const float r = 1.0f / sqrtf(ss / (float)C + eps);
+        if (ok && l == 0) rstd[row] = r;
+
+        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC], wv[VEC];
+            E::unpack(xr[k], v);
+            E::unpack(wr[k], wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= r;
+            E::round(v);  // y = normalised row in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+            if (ok && m.in[k]) store16_stream(po + k * LANES, E::pack(v));
+        }
+    }
+}
+
+template <typename T, int LANES, int CHUNKS>
+__global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
+    T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g, const T *__restrict__ x,
+    const T *__restrict__ w, const float *__restrict__ rstd, int64_t rows, int C) {
+    using G = PadGeom<T, LANES, CHUNKS>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, RPW = G::RPW;
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const LaneMask<G> m(l, C / VEC);
+
+    u32x4 wr[CHUNKS];
+    load_param<G>(wr, w, l, m);
+    float acc[1][CHUNKS][VEC];
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[0][k][j] = 0.0f;
+
+    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(wr);
+        const int64_t row = grp * RPW + sub;
+        const bool ok = row < rows;
+        u32x4 gr[CHUNKS], xr[CHUNKS];
+        load_row<G>(gr, g + row * C, l, ok, m);
+        load_row<G>(xr, x + row * C, l, ok, m);
+        const float r = ok ? rstd[row] : 0.0f;
+
+        // pass 1: gy = rnd(g*w) kept packed; row dot  sum_c gy * x
+        u32x4 gyp[CHUNKS];
+        float dot = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], wv[VEC], xv[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(wr[k], wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] *= wv[j];
+            gyp[k] = E::pack(gv);
+            E::unpack(gyp[k], gv);
+            E::unpack(xr[k], xv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) dot = fmaf(gv[j], xv[j], dot);
+        }
+        dot = group_sum<LANES>(dot);
+        // dx = r*(gy - xhat * mean_c(gy*xhat)) = gy*r + x*coef
+        const float coef = -((dot / (float)C) * r * r * r);
+        // the second pass unpacks the row again rather than holding pass 1's fp32 copies live
+        keep_packed(gr);
+        keep_packed(xr);
+        keep_packed(gyp);
+
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
+            E::unpack(gr[k], gv);
+            E::unpack(gyp[k], gy);
+            E::unpack(xr[k], xv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                o[j] = fmaf(xv[j], coef, gy[j] * r);
+                y[j] = xv[j] * r;
+            }
+            if (ok && m.in[k]) store16_stream(pd + k * LANES, E::pack(o));
+            E::round(y);  // y = normalised row in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
+            E::round(y);  // g*y materialised in the element type before the column sum
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[0][k][j] += y[j];
+        }
+    }
+    flush_partials_anywidth<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds, C, m);
+}
+
+// -------------------------------------------------------------------- AdaLN
+
+template <typename T, int LANES, int CHUNKS>
+__global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
+    T *__restrict__ out, float *__restrict__ mean, float *__restrict__ rstd, const T *__restrict__ x,
+    const T *__restrict__ scale, const T *__restrict__ shift, int64_t rows_per_sample, int blocks_per_sample,
+    int C, float eps) {
+    using G = PadGeom<T, LANES, CHUNKS>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, RPW = G::RPW;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const int64_t b = blockIdx.x / blocks_per_sample;  // sample this workgroup serves
+    const int slot = blockIdx.x % blocks_per_sample;
+    const LaneMask<G> m(l, C / VEC);
+
+    u32x4 tr[CHUNKS], hr[CHUNKS];
+    load_param<G>(tr, scale + b * C, l, m);
+    load_param<G>(hr, shift + b * C, l, m);
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {  // t = rnd(1 + scale)
+        float v[VEC];
+        E::unpack(tr[k], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
+        tr[k] = E::pack(v);
+    }
+
+    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
+    for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
+        keep_packed(tr);
+        keep_packed(hr);
+        const int64_t rs = grp * RPW + sub;
+        const bool ok = rs < rows_per_sample;
+        const int64_t row = b * rows_per_sample + rs;
+        u32x4 xr[CHUNKS];
+        load_row<G>(xr, x + row * C, l, ok, m);
+
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) s += v[j];
+        }
+        const float mu = group_sum<LANES>(s) / (float)C;
+        float q = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC];
+            E::unpack(xr[k], v);
+            if (m.in[k]) {  // padding must not count as (0 - mu)^2
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const float d = v[j] - mu;
+                    q = fmaf(d, d, q);
+                }
+            }
+        }
+        const float r = 1.0f / sqrtf(group_sum<LANES>(q) / (float)C + eps);
+        if (ok && l == 0) {
+            mean[row] = mu;
+            rstd[row] = r;
+        }
+
+        const float nmr = -(mu * r);
+        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float v[VEC], tv[VEC], hv[VEC];
+            E::unpack(xr[k], v);
+            E::unpack(tr[k], tv);
+            E::unpack(hr[k], hv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r
+            E::round(v);  // xn
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= tv[j];
+            E::round(v);  // xn * (1 + scale)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += hv[j];
+            if (ok && m.in[k]) store16_stream(po + k * LANES, E::pack(v));
+        }
+    }
+}
+
+template <typename T, int LANES, int CHUNKS>
+__global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
+    T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g, const T *__restrict__ x,
+    const T *__restrict__ scale, const float *__restrict__ mean, const float *__restrict__ rstd,
+    int64_t rows_per_sample, int blocks_per_sample, int C) {
+    using G = PadGeom<T, LANES, CHUNKS>;
+    using E = Elem<T>;
+    constexpr int VEC = G::VEC, RPW = G::RPW;
+    // the widest rows have no registers left for the modulation row: it is staged in LDS, in the
+    // area the final flush uses afterwards
+    constexpr bool kParamInRegs = CHUNKS <= 8;
+    // ... nor for gx = rnd(g*t) between the two passes: it is formed again (same rounding, same value)
+    constexpr bool kKeepGx = CHUNKS * VEC <= 64;
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int wave = wave_id_in_block();
+    const int64_t b = blockIdx.x / blocks_per_sample;
+    const int slot = blockIdx.x % blocks_per_sample;
+    const LaneMask<G> m(l, C / VEC);
+
+    auto one_plus = [](const u32x4 &raw) -> u32x4 {  // t = rnd(1 + scale)
+        float v[VEC];
+        E::unpack(raw, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
+        return E::pack(v);
+    };
+    u32x4 tr[kParamInRegs ? CHUNKS : 1];
+    u32x4 *lds_t = reinterpret_cast<u32x4 *>(lds);  // shares the flush area: dead before the flush starts
+    if constexpr (kParamInRegs) {
+        load_param<G>(tr, scale + b * C, l, m);
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) tr[k] = one_plus(tr[k]);
+    } else {
+        for (int i = threadIdx.x; i < C / VEC; i += kRowThreads)
+            lds_t[i] = one_plus(load16(reinterpret_cast<const u32x4 *>(scale + b * C) + i));
+        __syncthreads();
+    }
+
+    float acc[2][CHUNKS][VEC];  // [0] = dscale, [1] = dshift
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[s][k][j] = 0.0f;
+
+    const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
+    const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
+    for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
+        if constexpr (kParamInRegs) keep_packed(tr);
+        const int64_t rs = grp * RPW + sub;
+        const bool ok = rs < rows_per_sample;
+        const int64_t row = b * rows_per_sample + rs;
+        u32x4 gr[CHUNKS], xr[CHUNKS];
+        load_row<G>(gr, g + row * C, l, ok, m);
+        load_row<G>(xr, x + row * C, l, ok, m);
+        const float r = ok ? rstd[row] : 0.0f;
+        const float mu = ok ? mean[row] : 0.0f;
+        const float nmr = -(mu * r);  // xhat = x*r + nmr
+
+        auto gx_of = [&](int k) -> u32x4 {  // rnd(g * t) for access k, in the element type
+            float gv[VEC], tv[VEC];
+            E::unpack(gr[k], gv);
+            if constexpr (kParamInRegs)
+                E::unpack(tr[k], tv);
+            else
+                E::unpack(m.in[k] ? lds_t[k * LANES + l] : u32x4{0, 0, 0, 0}, tv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] *= tv[j];
+            return E::pack(gv);
+        };
+        // pass 1: gx = rnd(g*t); s1 = sum_c gx; s2 = sum_c gx * xhat
+        u32x4 gxp[kKeepGx ? CHUNKS : 1];
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            const u32x4 gxk = gx_of(k);
+            if constexpr (kKeepGx) gxp[k] = gxk;
+            // padding: g = 0 there, so gx = 0 and neither sum sees xhat = nmr
+            if constexpr (kIsBf16<T>) {
+                // straight from the packed pairs; s2 holds sum_c gx * x here, turned into sum_c gx * xhat below
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s1 = dot2_bf16(gxk[i], kBf16OnesPair, s1);
+                    s2 = dot2_bf16(gxk[i], xr[k][i], s2);
+                }
+            } else {
+                float gv[VEC], xv[VEC];
+                E::unpack(gxk, gv);
+                E::unpack(xr[k], xv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    s1 += gv[j];
+                    s2 = fmaf(gv[j], fmaf(xv[j], r, nmr), s2);
+                }
+            }
+        }
+        s1 = group_sum<LANES>(s1);
+        s2 = group_sum<LANES>(s2);
+        if constexpr (kIsBf16<T>) s2 = r * (s2 - mu * s1);
+        const float m1 = s1 / (float)C, m2 = s2 / (float)C;
+        // dx = r*(gx - m1 - xhat*m2) = r*gx + x*K1 + K0
+        const float k1 = -(r * m2), k0 = -(r * m1);
+        const float K1 = k1 * r;
+        const float K0 = fmaf(k1, nmr, k0);
+        // the second pass unpacks the row again rather than holding pass 1's fp32 copies live
+        keep_packed(gr);
+        keep_packed(xr);
+        if constexpr (kKeepGx) keep_packed(gxp);
+
+        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
+            E::unpack(gr[k], gv);
+            if constexpr (kKeepGx)
+                E::unpack(gxp[k], gx);
+            else
+                E::unpack(gx_of(k), gx);
+            E::unpack(xr[k], xv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
+                xn[j] = fmaf(xv[j], r, nmr);
+                acc[1][k][j] += gv[j];
+            }
+            if (ok && m.in[k]) store16_stream(pd + k * LANES, E::pack(o));
+            E::round(xn);  // the normalised row in the element type
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
+            E::round(xn);  // g*xn materialised in the element type before the column sum
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[0][k][j] += xn[j];
+        }
+    }
+    if constexpr (!kParamInRegs) __syncthreads();  // every wavefront is done reading lds_t
+    flush_partials_anywidth<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds, C, m);
+}
+
+// ---------------------------------------------------------------- dispatch
+
+constexpr int kMaxPieces = 1024;  // 16-byte accesses per row: 64 lanes x 16
+
+bool anywidth_supported(int64_t cols, int dtype) {
+    if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F32 && dtype != TT_NORM_F16) return false;
+    const int vec = 16 / (int)elem_bytes(dtype);
+    return cols > 0 && cols % vec == 0 && cols / vec <= kMaxPieces;
+}
+
+// The smallest instantiated geometry that holds `pieces` accesses.
+struct GeomChoice {
+    int lanes, chunks;
+};
+static GeomChoice choose_geometry(int pieces) {
+    if (pieces <= 16) return {16, 1};
+    if (pieces <= 32) return {32, 1};
+    const int need = (pieces + 63) / 64;
+    for (int c : {1, 2, 3, 4, 6, 8, 12, 16})
+        if (need <= c) return {64, c};
+    return {0, 0};
+}
+
+// Calls F<T, LANES, CHUNKS>::run(args...) for the run-time (dtype, geometry).
+#define TTN_ANYWIDTH_GEOMS(X, T) \
+    X(T, 16, 1) X(T, 32, 1) X(T, 64, 1) X(T, 64, 2) X(T, 64, 3) X(T, 64, 4) X(T, 64, 6) X(T, 64, 8) X(T, 64, 12) X(T, 64, 16)
+
+template <template <typename, int, int> class F, typename... Args>
+static int dispatch(int dtype, GeomChoice gc, Args... args) {
+#define TTN_TRY(T, L, K) \
+    if (gc.lanes == L && gc.chunks == K) return F<T, L, K>::run(args...);
+    if (dtype == TT_NORM_BF16) {
+        TTN_ANYWIDTH_GEOMS(TTN_TRY, bf16_t)
+    } else if (dtype == TT_NORM_F16) {
+        TTN_ANYWIDTH_GEOMS(TTN_TRY, f16_t)
+    } else {
+        TTN_ANYWIDTH_GEOMS(TTN_TRY, float)
+    }
+#undef TTN_TRY
+    return fail(TT_NORM_EUNSUPPORTED, "no kernel geometry for %d lanes x %d accesses", gc.lanes, gc.chunks);
+}
+
+// Launch policy.  Forward: narrow rows (one access per lane) use a persistent grid of 16 workgroups
+// per compute unit, wider rows one row per wavefront.  Backward is persistent (column sums live in
+// registers); the grid shrinks as rows widen so that each compute unit keeps about the same number
+// of bytes in flight.
+constexpr int kOneShotAny = 1 << 20;
+static int fwd_blocks_per_cu(int chunks) { return chunks == 1 ? 16 : kOneShotAny; }
+static int bwd_blocks_per_cu(int chunks) { return chunks >= 6 ? 1 : (chunks >= 3 ? 2 : (chunks == 2 ? 3 : 6)); }
+
+static GeomChoice geometry_for(int64_t cols, int dtype) {
+    return choose_geometry((int)(cols / (16 / (int)elem_bytes(dtype))));
+}
+
+// Grid for (batch, rows_per_sample) under geometry gc; status != OK on failure.
+static int plan_for(RowPlan *plan, int64_t batch, int64_t rows_per_sample, GeomChoice gc, bool backward) {
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    *plan = make_row_plan(batch, rows_per_sample, kWaveSize / gc.lanes,
+                          backward ? bwd_blocks_per_cu(gc.chunks) : fwd_blocks_per_cu(gc.chunks), cus);
+    if (plan->blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "grid too large");
+    return TT_NORM_OK;
+}
+
+template <typename T, int LANES, int CHUNKS>
+struct RmsFwd {
+    static int run(const RowPlan &p, void *out, float *rstd, const void *x, const void *w, int64_t rows, int C,
+                   double eps, hipStream_t stream) {
+        RowKernelProfile prof(stream);
+        anywidth_rmsnorm_fwd_kernel<T, LANES, CHUNKS><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+            (T *)out, rstd, (const T *)x, (const T *)w, rows, C, (float)eps);
+        return TT_NORM_OK;
+    }
+};
+
+template <typename T, int LANES, int CHUNKS>
+struct RmsBwd {
+    static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *w,
+                   const float *rstd, int64_t rows, int C, hipStream_t stream) {
+        RowKernelProfile prof(stream);
+        anywidth_rmsnorm_bwd_kernel<T, LANES, CHUNKS>
+            <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)C * sizeof(float), stream>>>(
+                (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)w, rstd, rows, C);
+        return TT_NORM_OK;
+    }
+};
+
+template <typename T, int LANES, int CHUNKS>
+struct AdalnFwd {
+    static int run(const RowPlan &p, void *out, float *mean, float *rstd, const void *x, const void *scale,
+                   const void *shift, int64_t rows_per_sample, int C, double eps, hipStream_t stream) {
+        RowKernelProfile prof(stream);
+        anywidth_adaln_fwd_kernel<T, LANES, CHUNKS><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+            (T *)out, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift, rows_per_sample,
+            p.blocks_per_sample, C, (float)eps);
+        return TT_NORM_OK;
+    }
+};
+
+template <typename T, int LANES, int CHUNKS>
+struct AdalnBwd {
+    static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *scale,
+                   const float *mean, const float *rstd, int64_t rows_per_sample, int C, hipStream_t stream) {
+        RowKernelProfile prof(stream);
+        anywidth_adaln_bwd_kernel<T, LANES, CHUNKS>
+            <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)2 * C * sizeof(float), stream>>>(
+                (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)scale, mean, rstd, rows_per_sample,
+                p.blocks_per_sample, C);
+        return TT_NORM_OK;
+    }
+};
+
+int anywidth_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
+                             double eps, int dtype, hipStream_t stream) {
+    if (rows == 0) return TT_NORM_OK;
+    const GeomChoice gc = geometry_for(cols, dtype);
+    RowPlan p;
+    int st = plan_for(&p, 1, rows, gc, false);
+    if (st != TT_NORM_OK) return st;
+    st = dispatch<RmsFwd>(dtype, gc, p, out, rstd, x, w, rows, (int)cols, eps, stream);
+    return st != TT_NORM_OK ? st : check_launch("rmsnorm forward launch");
+}
+
+static size_t backward_scratch(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, int nsets) {
+    if (batch <= 0 || rows_per_sample <= 0 || !anywidth_supported(cols, dtype)) return 0;
+    RowPlan p;
+    if (plan_for(&p, batch, rows_per_sample, geometry_for(cols, dtype), true) != TT_NORM_OK) return 0;
+    return (size_t)p.blocks * nsets * cols * sizeof(float);
+}
+
+size_t anywidth_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
+    return backward_scratch(1, rows, cols, dtype, 1);
+}
+
+int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
+                              const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
+                              size_t ws_bytes, hipStream_t stream) {
+    if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, nullptr, 1, 0, cols, cols, dtype, stream);
+    const GeomChoice gc = geometry_for(cols, dtype);
+    RowPlan p;
+    int st = plan_for(&p, 1, rows, gc, true);
+    if (st != TT_NORM_OK) return st;
+    const size_t need = (size_t)p.blocks * cols * sizeof(float);
+    if (!ws || ws_bytes < need)
+        return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
+    st = dispatch<RmsBwd>(dtype, gc, p, dx, ws, g, x, w, rstd, rows, (int)cols, stream);
+    if (st != TT_NORM_OK) return st;
+    st = check_launch("rmsnorm backward launch");
+    if (st != TT_NORM_OK) return st;
+    return launch_colreduce(dw, nullptr, nullptr, (const float *)ws, 1, p.blocks_per_sample, cols, cols, dtype,
+                            stream);
+}
+
+int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                           const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
+                           int dtype, hipStream_t stream) {
+    if (rows_per_sample == 0) return TT_NORM_OK;
+    const GeomChoice gc = geometry_for(cols, dtype);
+    RowPlan p;
+    int st = plan_for(&p, batch, rows_per_sample, gc, false);
+    if (st != TT_NORM_OK) return st;
+    st = dispatch<AdalnFwd>(dtype, gc, p, out, mean, rstd, x, scale, shift, rows_per_sample, (int)cols, eps, stream);
+    return st != TT_NORM_OK ? st : check_launch("adaln forward launch");
+}
+
+size_t anywidth_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
+    return backward_scratch(batch, rows_per_sample, cols, dtype, 2);
+}
+
+int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x,
+                            const void *scale, const float *mean, const float *rstd, int64_t batch,
+                            int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                            hipStream_t stream) {
+    if (rows_per_sample == 0)
+        return launch_colreduce(dscale, dshift, nullptr, nullptr, batch, 0, cols, 2 * cols, dtype, stream);
+    const GeomChoice gc = geometry_for(cols, dtype);
+    RowPlan p;
+    int st = plan_for(&p, batch, rows_per_sample, gc, true);
+    if (st != TT_NORM_OK) return st;
+    const size_t need = (size_t)p.blocks * 2 * cols * sizeof(float);
+    if (!ws || ws_bytes < need)
+        return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
+    st = dispatch<AdalnBwd>(dtype, gc, p, dx, ws, g, x, scale, mean, rstd, rows_per_sample, (int)cols, stream);
+    if (st != TT_NORM_OK) return st;
+    st = check_launch("adaln backward launch");
+    if (st != TT_NORM_OK) return st;
+    return launch_colreduce(dscale, dshift, nullptr, (const float *)ws, batch, p.blocks_per_sample, cols, 2 * cols,
+                            dtype, stream);
+}
+
+}  // namespace ttn

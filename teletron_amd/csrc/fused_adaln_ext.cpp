@@ -196,7 +196,8 @@ PYBIND11_MODULE(fused_adaln, m) {
           "AdaLN backward kernel (from the saved input and statistics)");
     m.def("supported", [](int64_t cols, const torch::Tensor &like) {
         return tt_norm_supported(cols, like.scalar_type() == at::kBFloat16 ? TT_NORM_BF16
-                                       : like.scalar_type() == at::kFloat  ? TT_NORM_F32 : -1) != 0;
+                                       : like.scalar_type() == at::kFloat  ? TT_NORM_F32
+                                       : like.scalar_type() == at::kHalf   ? TT_NORM_F16 : -1) != 0;
     }, "whether the kernels are built for this column count and dtype");
 }
 

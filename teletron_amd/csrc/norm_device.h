@@ -25,8 +25,13 @@ namespace ttn {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
-// Storage-only tag for bf16 elements (arithmetic is always fp32).
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// Storage-only tags for 2-byte elements (arithmetic is always fp32).
 struct bf16_t {
+    uint16_t bits;
+};
+struct f16_t {
     uint16_t bits;
 };
 
@@ -83,6 +88,36 @@ struct Elem<bf16_t> {
     }
     // Round every value to bf16 and back: the eager graph materialises this
     // tensor in bf16 at this point.
+    static __device__ __forceinline__ void round(float (&v)[8]) {
+        u32x4 r = pack(v);
+        unpack(r, v);
+    }
+};
+
+// IEEE half: conversions are the hardware's (v_cvt_f32_f16 exact, v_cvt_f16_f32 in the default
+// round-to-nearest-even mode, subnormals kept).
+template <>
+struct Elem<f16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f16x2_t h = __builtin_bit_cast(f16x2_t, (uint32_t)r[i]);
+            v[2 * i] = (float)h[0];
+            v[2 * i + 1] = (float)h[1];
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f16x2_t h;
+            h[0] = (_Float16)v[2 * i];
+            h[1] = (_Float16)v[2 * i + 1];
+            r[i] = __builtin_bit_cast(uint32_t, h);
+        }
+        return r;
+    }
     static __device__ __forceinline__ void round(float (&v)[8]) {
         u32x4 r = pack(v);
         unpack(r, v);

@@ -20,7 +20,12 @@ int current_device_cus(int *status);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-inline size_t elem_bytes(int dtype) { return dtype == TT_NORM_BF16 ? 2 : 4; }
+inline size_t elem_bytes(int dtype) { return dtype == TT_NORM_F32 ? 4 : 2; }
+
+// (cols, dtype) the tuned kernels of rmsnorm.hip / adaln.hip are built for.
+inline bool tuned_shape(int64_t cols, int dtype) {
+    return (cols == 128 || cols == 3072) && (dtype == TT_NORM_BF16 || dtype == TT_NORM_F32);
+}
 
 // Checks the last launch on this thread; returns TT_NORM_OK or TT_NORM_EHIP.
 int check_launch(const char *what);
@@ -62,5 +67,24 @@ RowPlan make_row_plan(int64_t batch, int64_t rows_per_sample, int rows_per_wave,
 int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, int64_t batch,
                      int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
                      hipStream_t stream);
+
+// ---- any-width kernels (anywidth.hip): every other supported (cols, dtype) -----
+// Native contract only (saved input + row statistics); same argument meaning as the
+// C-ABI entry points that forward to them.
+bool anywidth_supported(int64_t cols, int dtype);
+int anywidth_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
+                             double eps, int dtype, hipStream_t stream);
+size_t anywidth_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
+                              const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
+                              size_t ws_bytes, hipStream_t stream);
+int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                           const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
+                           int dtype, hipStream_t stream);
+size_t anywidth_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype);
+int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x,
+                            const void *scale, const float *mean, const float *rstd, int64_t batch,
+                            int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                            hipStream_t stream);
 
 }  // namespace ttn

@@ -95,6 +95,10 @@ template <>
 __device__ __forceinline__ void store_scalar<bf16_t>(bf16_t *p, float v) {
     p->bits = (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu);
 }
+template <>
+__device__ __forceinline__ void store_scalar<f16_t>(f16_t *p, float v) {
+    p->bits = __builtin_bit_cast(uint16_t, (_Float16)v);
+}
 
 template <typename T>
 __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
@@ -140,6 +144,9 @@ int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, i
     if (dtype == TT_NORM_BF16)
         colreduce_kernel<bf16_t><<<g, blk, 0, stream>>>((bf16_t *)out0, (bf16_t *)out1, (bf16_t *)out2, partial,
                                                         blocks_per_sample, (int)C, (int)ncols, col_blocks);
+    else if (dtype == TT_NORM_F16)
+        colreduce_kernel<f16_t><<<g, blk, 0, stream>>>((f16_t *)out0, (f16_t *)out1, (f16_t *)out2, partial,
+                                                       blocks_per_sample, (int)C, (int)ncols, col_blocks);
     else
         colreduce_kernel<float><<<g, blk, 0, stream>>>((float *)out0, (float *)out1, (float *)out2, partial,
                                                        blocks_per_sample, (int)C, (int)ncols, col_blocks);
@@ -181,7 +188,7 @@ const char *tt_norm_status_string(int status) {
     switch (status) {
         case TT_NORM_OK: return "ok";
         case TT_NORM_EINVAL: return "invalid argument";
-        case TT_NORM_EUNSUPPORTED: return "unsupported cols/dtype";
+        case TT_NORM_EUNSUPPORTED: return "unsupported cols/dtype for this entry point";
         case TT_NORM_EALIGN: return "pointer not 16-byte aligned";
         case TT_NORM_EWORKSPACE: return "workspace missing or too small";
         case TT_NORM_EHIP: return "HIP runtime error";
@@ -192,9 +199,10 @@ const char *tt_norm_status_string(int status) {
 const char *tt_norm_last_error(void) { return g_last_error; }
 
 int tt_norm_supported(int64_t cols, int dtype) {
-    if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F32) return 0;
-    return (cols == 128 || cols == 3072) ? 1 : 0;
+    return (tuned_shape(cols, dtype) || anywidth_supported(cols, dtype)) ? 1 : 0;
 }
+
+int tt_norm_tuned(int64_t cols, int dtype) { return tuned_shape(cols, dtype) ? 1 : 0; }
 
 int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event) {
     if ((start_event == nullptr) != (stop_event == nullptr))

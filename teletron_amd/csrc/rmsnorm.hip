@@ -345,12 +345,17 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
     return launch_colreduce(dw, nullptr, nullptr, (const float *)ws, 1, p.blocks_per_sample, C, C, dtype, stream);
 }
 
+// tuned_only: the entry point exists for the tuned shapes only (reference-contract and strided forms).
 static int check_rms_args(const char *who, int64_t rows, int64_t cols, int dtype,
-                          std::initializer_list<const void *> ptrs) {
+                          std::initializer_list<const void *> ptrs, bool tuned_only = false) {
     if (rows < 0 || cols <= 0) return fail(TT_NORM_EINVAL, "%s: rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
-    if (!tt_norm_supported(cols, dtype))
-        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (built for cols 128/3072, bf16/fp32)", who,
+    if (tuned_only && !tuned_shape(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072, bf16/fp32)", who,
                     (long long)cols, dtype);
+    if (!tt_norm_supported(cols, dtype))
+        return fail(TT_NORM_EUNSUPPORTED,
+                    "%s: cols=%lld dtype=%d (cols must be a multiple of 16 bytes of elements, at most 8192 "
+                    "two-byte or 4096 four-byte; dtype bf16, fp16 or fp32)", who, (long long)cols, dtype);
     if (rows == 0) return TT_NORM_OK;  // empty input: nothing is dereferenced
     for (const void *p : ptrs) {
         if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
@@ -381,6 +386,8 @@ int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight
     int st = check_rms_args("tt_rmsnorm_forward", rows, cols, dtype, {out, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward: null rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_rmsnorm_forward(out, rstd, x, weight, rows, cols, eps, dtype, (hipStream_t)stream);
 #define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, DenseRows{rows}, rows, eps, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
@@ -388,6 +395,7 @@ int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight
 
 size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
     if (rows <= 0 || !tt_norm_supported(cols, dtype)) return 0;
+    if (!tuned_shape(cols, dtype)) return anywidth_rmsnorm_backward_workspace_bytes(rows, cols, dtype);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return 0;
@@ -402,6 +410,9 @@ int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x
     int st = check_rms_args("tt_rmsnorm_backward", rows, cols, dtype, {dx, dout, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_rmsnorm_backward(dx, dweight, dout, x, weight, rstd, rows, cols, dtype, workspace,
+                                         workspace_bytes, (hipStream_t)stream);
 #define CALL(T, C)                                                                                  \
     return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, DenseRows{rows}, rows, dtype, \
                                            workspace, workspace_bytes, (hipStream_t)stream)
@@ -412,7 +423,7 @@ int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x
 int tt_rmsnorm_backward_from_out(void *dx, void *dweight, const void *dout, const void *out,
                                  const void *weight, const float *rstd, int64_t rows, int64_t cols,
                                  int dtype, void *workspace, size_t workspace_bytes, void *stream) {
-    int st = check_rms_args("tt_rmsnorm_backward_from_out", rows, cols, dtype, {dx, dout, out, weight});
+    int st = check_rms_args("tt_rmsnorm_backward_from_out", rows, cols, dtype, {dx, dout, out, weight}, true);
     if (st != TT_NORM_OK) return st;
     if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_from_out: null dweight/rstd");
 #define CALL(T, C)                                                                                   \
@@ -442,7 +453,7 @@ int tt_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void
     int st = check_strided("tt_rmsnorm_forward_strided", n0, n1, n2, cols, dtype, xs, "x");
     if (st != TT_NORM_OK) return st;
     const int64_t rows = n0 * n1 * n2;
-    st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight});
+    st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight}, true);
     if (st != TT_NORM_OK) return st;
     if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward_strided: null rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, 0, 0, 0};
@@ -461,7 +472,7 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
     if (st == TT_NORM_OK) st = check_strided("tt_rmsnorm_backward_strided", n0, n1, n2, cols, dtype, ds, "dx");
     if (st != TT_NORM_OK) return st;
     const int64_t rows = n0 * n1 * n2;
-    st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight});
+    st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight}, true);
     if (st != TT_NORM_OK) return st;
     if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_strided: null dweight/rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, dxs0, dxs1, dxs2};

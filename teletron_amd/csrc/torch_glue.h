@@ -14,7 +14,8 @@ namespace ttn_glue {
 inline int dtype_code(const at::Tensor &t, const char *name) {
     if (t.scalar_type() == at::kBFloat16) return TT_NORM_BF16;
     if (t.scalar_type() == at::kFloat) return TT_NORM_F32;
-    TORCH_CHECK(false, name, ": expected a bfloat16 or float32 tensor, got ", t.scalar_type());
+    if (t.scalar_type() == at::kHalf) return TT_NORM_F16;
+    TORCH_CHECK(false, name, ": expected a bfloat16, float16 or float32 tensor, got ", t.scalar_type());
 }
 
 inline void check_dense_on(const at::Tensor &t, const at::Device &dev, const char *name) {

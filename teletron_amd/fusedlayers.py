@@ -43,7 +43,24 @@ except ImportError as exc:  # pragma: no cover - exercised only on an unbuilt tr
     log.warning("fused_adaln / fused_rmsnorm extensions not importable (%s); "
                 "build them with `python -m teletron_amd.build`.", exc)
 
-SUPPORTED_COLS = (128, 3072)
+TUNED_COLS = (128, 3072)  # the reference's two shapes; strided views and the gated op need these
+_ELEM_BYTES = {torch.bfloat16: 2, torch.float16: 2, torch.float32: 4}
+_MAX_PIECES = 1024  # 16-byte pieces per row the kernels are built for
+
+
+def cols_supported(cols: int, dtype: torch.dtype) -> bool:
+    """Whether the fused kernels take rows of `cols` elements of `dtype`: whole 16-byte pieces,
+    at most 8192 two-byte or 4096 four-byte columns, bf16 / fp16 / fp32."""
+    size = _ELEM_BYTES.get(dtype)
+    if size is None or cols <= 0:
+        return False
+    vec = 16 // size
+    return cols % vec == 0 and cols // vec <= _MAX_PIECES
+
+
+def _unsupported(cols: int, dtype: torch.dtype) -> str:
+    return (f"unsupported cols {cols} for {dtype}: rows must be whole 16-byte pieces, at most 8192 two-byte "
+            f"or 4096 four-byte columns, dtype bfloat16, float16 or float32")
 
 
 def fused_kernels_available() -> bool:
@@ -98,9 +115,10 @@ class AdaLNModelFunction(Function):
         x = _aligned_contiguous(x)
         scale_c = scale.contiguous()
         shift_c = shift.contiguous()
-        if cols not in SUPPORTED_COLS or x.numel() % cols != 0:
-            raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols} "
-                             f"or unsupported cols (supported: {SUPPORTED_COLS})")
+        if x.numel() % cols != 0:
+            raise ValueError(f"Input tensor size {x.numel()} not divisible by cols {cols}")
+        if not cols_supported(cols, x.dtype):
+            raise ValueError(_unsupported(cols, x.dtype))
         rows = x.numel() // cols
         if scale_c.numel() % cols != 0 or shift_c.numel() != scale_c.numel():
             raise ValueError(f"scale/shift sizes {scale_c.numel()}/{shift_c.numel()} do not match cols {cols}")
@@ -260,8 +278,8 @@ class _AdaLNZeroBase(nn.Module):
         self.fused_kernels = bool(fused_kernels)
         self.embedding_dim = embedding_dim
         if self.fused_kernels:
-            if embedding_dim not in SUPPORTED_COLS:
-                raise ValueError(f"fused_kernels=True needs embedding_dim in {SUPPORTED_COLS}, got {embedding_dim}")
+            if not cols_supported(embedding_dim, torch.float32):  # the strictest element size
+                raise ValueError(f"fused_kernels=True: {_unsupported(embedding_dim, torch.float32)}")
             _require_extension(fused_adaln, "fused_adaln")
             self.adaLN = AdaLNCustom(embedding_dim, eps=1e-6)
         elif norm_type == "layer_norm":
@@ -348,12 +366,14 @@ class RMSNormModelFunction(Function):
     def forward(ctx, x, weight, epsilon, cols):
         ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
         _require_gpu(x, "RMSNormModelFunction")
-        if cols not in SUPPORTED_COLS or x.numel() % cols != 0:
-            raise ValueError(f"Input size {x.numel()} not divisible by cols {cols} or unsupported cols value "
-                             f"(supported: {SUPPORTED_COLS})")
+        if x.numel() % cols != 0:
+            raise ValueError(f"Input size {x.numel()} not divisible by cols {cols}")
+        if not cols_supported(cols, x.dtype):
+            raise ValueError(_unsupported(cols, x.dtype))
         if weight.numel() != cols:
             raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
-        strided = x.shape[-1] == cols and _strided_rows_ok(x)
+        tuned = cols in TUNED_COLS and x.dtype in (torch.bfloat16, torch.float32)
+        strided = tuned and x.shape[-1] == cols and _strided_rows_ok(x)
         if not strided:
             x = _aligned_contiguous(x)
         w = weight.contiguous()
@@ -403,7 +423,7 @@ class RMSNorm(nn.Module):
         return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps)
 
     def forward(self, x):
-        if fused_kernels_requested() and self.hidden_size in SUPPORTED_COLS:
+        if fused_kernels_requested() and cols_supported(self.hidden_size, x.dtype):
             return RMSNormModelFunction.apply(x, self.weight, self.eps, self.hidden_size)
         return self._norm(x.float()).type_as(x) * self.weight
 

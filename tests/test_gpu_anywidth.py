@@ -1,0 +1,163 @@
+"""GPU parity of the any-width kernels (rows of any whole number of 16-byte pieces, bf16 / fp16 /
+fp32) through the C ABI, against the eager oracle.  Same bars as tests/test_gpu_parity.py:
+forward 16-bit: >= 99.9 % bit-identical, <= 1 ulp except excused cancellation cases; forward fp32
+rel 1e-5; gradients 16-bit |got - want| <= 1e-3 + 1e-2 |want|; gradients fp32 rel 1e-4."""
+import pytest
+import torch
+
+from oracle import norm_oracle as O
+
+pytestmark = pytest.mark.gpu
+EPS = 1e-6
+
+BF, HF, F32 = torch.bfloat16, torch.float16, torch.float32
+# (cols, rows, dtype): every kernel geometry (16 / 32 lanes; 1, 2, 3, 4, 6, 8, 12, 16 accesses per lane),
+# full and ragged last accesses, row counts that do not fill the last wavefront
+RMS_CASES = [
+    (8, 5, BF), (64, 1001, BF), (96, 130, BF), (128, 77, HF), (200, 513, BF), (256, 4099, BF), (512, 300, BF),
+    (768, 257, BF), (1000, 50, BF), (1024, 1000, BF), (1536, 333, HF), (2048, 77, BF), (2560, 65, BF),
+    (3072, 300, HF), (3080, 33, BF), (4096, 129, BF), (5120, 130, BF), (6144, 70, HF), (8192, 66, BF),
+    (8192, 9, HF), (4, 3, F32), (64, 100, F32), (256, 1000, F32), (1000, 77, F32), (2048, 129, F32), (4096, 40, F32),
+]
+ADALN_CASES = [
+    (1, 5, 8, BF), (3, 333, 64, BF), (2, 65, 96, HF), (2, 1001, 256, BF), (4, 100, 512, BF), (1, 257, 1000, BF),
+    (2, 130, 1024, HF), (3, 77, 1536, BF), (2, 300, 2048, BF), (5, 33, 3072, HF), (2, 65, 4096, BF),
+    (2, 130, 5120, BF), (3, 40, 6144, BF), (2, 35, 6144, HF), (2, 66, 8192, BF), (1, 9, 8192, HF),
+    (2, 50, 64, F32), (3, 100, 1000, F32), (2, 40, 4096, F32),
+]
+
+
+@pytest.fixture(scope="module")
+def capi(gpu_device):
+    from teletron_amd import capi as c
+    c.lib()
+    return c
+
+
+def fwd_16bit_ok(got, want, excuse, what):
+    rep = O.compare_bf16_ulp(got.cpu(), want, excuse_abs=excuse)
+    assert rep.n_gt1 == 0, (what, rep)
+    assert rep.n_excused <= max(2, 1e-4 * rep.n), (what, rep)
+    assert rep.frac_exact >= 0.999 or rep.n - rep.n_exact <= 2, (what, rep)
+
+
+def grad_ok(got, want, what, allow=0.0):
+    if want.dtype == F32:
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-5, msg=what)
+    else:
+        assert O.frac_outside(got.cpu(), want, 1e-2, 1e-3) <= allow, what
+
+
+def colsum_ok(got, want, terms, dim, what):
+    """Column sums.  fp32: within 1e-4 of the column's L1 mass.  16-bit: the gradient bar on all but
+    1e-4 of columns, and every column within 1e-2 |want| + 2^-8 * L2 mass (a term that flips by one ulp
+    in one implementation moves a cancelling column by more than the absolute part of the bar)."""
+    if want.dtype == F32:
+        l1 = terms.abs().sum(dim).reshape(want.shape)
+        assert ((got.cpu() - want).abs() <= 1e-4 * l1 + 1e-5).all(), what
+    else:
+        assert O.frac_outside(got.cpu(), want, 1e-2, 1e-3) <= 1e-4, what
+        assert O.colsum_outside(got.cpu(), want, terms, dim, ulp=2.0 ** -8) == 0, what
+
+
+@pytest.mark.parametrize("cols,rows,dtype", RMS_CASES)
+def test_rmsnorm_any_width_vs_eager(capi, gpu_device, cols, rows, dtype):
+    d = O.make_rmsnorm_inputs((rows,), cols, dtype, seed=500 + cols % 101 + rows % 7)
+    want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    x, w, g = (d[k].to(gpu_device) for k in ("x", "weight", "grad"))
+    out, rstd = capi.rmsnorm_forward(x, w, EPS)
+    if dtype == F32:
+        torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-6)
+    else:
+        fwd_16bit_ok(out, want_out, O.rmsnorm_excuse(want_out), "out")
+    _, want_r = O.staged_rmsnorm_fwd(d["x"], d["weight"])
+    torch.testing.assert_close(rstd.cpu(), want_r.reshape(-1), rtol=2e-6, atol=0)
+    dx, dw = capi.rmsnorm_backward(g, x, w, rstd)
+    grad_ok(dx, want_dx, "dx")
+    colsum_ok(dw, want_dw, d["grad"].float() * want_out.float(), 0, "dweight")
+    dx2, dw2 = capi.rmsnorm_backward(g, x, w, rstd)
+    assert torch.equal(dx, dx2) and torch.equal(dw, dw2)      # fixed-order reduction
+
+
+@pytest.mark.parametrize("batch,seq,cols,dtype", ADALN_CASES)
+def test_adaln_any_width_vs_eager(capi, gpu_device, batch, seq, cols, dtype):
+    d = O.make_adaln_inputs(batch, seq, cols, dtype, seed=600 + cols % 103 + seq % 5, sigma=1.5)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    x, sc, sh, g = (d[k].to(gpu_device) for k in ("x", "scale", "shift", "grad"))
+    out, mean, rstd = capi.adaln_forward(x, sc, sh, EPS)
+    if dtype == F32:
+        torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-5)
+    else:
+        fwd_16bit_ok(out, want_out, O.adaln_excuse(d["x"], d["scale"], d["shift"], want_out), "out")
+    _, want_mu, want_r = O.staged_adaln_fwd(d["x"], d["scale"], d["shift"])
+    torch.testing.assert_close(rstd.cpu(), want_r.reshape(-1), rtol=4e-6, atol=0)
+    torch.testing.assert_close(mean.cpu(), want_mu.reshape(-1), rtol=0, atol=2e-6)
+    dx, ds, dh = capi.adaln_backward(g, x, sc, mean, rstd)
+    if dtype == F32:
+        grad_ok(dx, want_dx, "dx")
+    else:  # narrow rows: the bound scales with the terms the backward adds (see adaln_dx_terms)
+        terms = O.adaln_dx_terms(d["x"], d["scale"], d["grad"])
+        assert O.frac_outside(dx.cpu(), want_dx, 1e-2, 1e-3, magnitude=terms) <= 1e-4, "dx"
+    xn = torch.nn.functional.layer_norm(d["x"].float(), (cols,), None, None, EPS)
+    colsum_ok(ds, want_ds, d["grad"].float() * xn, 1, "dscale")
+    colsum_ok(dh, want_dh, d["grad"].float(), 1, "dshift")
+    again = capi.adaln_backward(g, x, sc, mean, rstd)
+    assert all(torch.equal(a, b) for a, b in zip((dx, ds, dh), again))
+
+
+def test_tuned_and_any_width_kernels_agree_bitwise_on_statistics(capi, gpu_device):
+    """3072 columns in fp16 run the any-width kernels; the same values held in bf16-exact form must give
+    the same row statistics as the tuned bf16 kernels (same sums in the same lane order)."""
+    d = O.make_adaln_inputs(2, 131, 3072, BF, seed=7)
+    x = d["x"].to(gpu_device)
+    sc, sh = d["scale"].to(gpu_device), d["shift"].to(gpu_device)
+    _, mean_t, rstd_t = capi.adaln_forward(x, sc, sh, EPS)
+    _, mean_a, rstd_a = capi.adaln_forward(x.half(), sc.half(), sh.half(), EPS)   # N(0, 1.5): exact in fp16 too
+    exact = (x.half().float() == x.float()).all(dim=-1).reshape(-1)
+    assert exact.float().mean() > 0.5
+    torch.testing.assert_close(mean_a[exact], mean_t[exact], rtol=0, atol=1e-6)
+    torch.testing.assert_close(rstd_a[exact], rstd_t[exact], rtol=2e-6, atol=0)
+
+
+def test_unsupported_widths_and_entry_points(capi, gpu_device):
+    mk = lambda *shape, dt=BF: torch.zeros(*shape, device=gpu_device, dtype=dt)
+    for cols, dt in ((100, BF), (8200, BF), (4100, F32), (6, F32)):
+        with pytest.raises(capi.NormError) as e:
+            capi.rmsnorm_forward(mk(4, cols, dt=dt), mk(cols, dt=dt), EPS)
+        assert e.value.status == 2
+    # reference-contract and strided entry points exist for the tuned shapes only
+    with pytest.raises(capi.NormError) as e:
+        capi.rmsnorm_backward(mk(4, 256), mk(4, 256), mk(256), torch.zeros(4, device=gpu_device), from_out=True)
+    assert e.value.status == 2
+    with pytest.raises(capi.NormError) as e:
+        capi.adaln_forward(mk(1, 4, 256), mk(1, 256), mk(1, 256), EPS, want_xnorm=True)
+    assert e.value.status == 2
+    # zero rows at a non-tuned width: no-op forward, zero parameter gradients
+    out, rstd = capi.rmsnorm_forward(mk(0, 512, dt=HF), mk(512, dt=HF), EPS)
+    dx, dw = capi.rmsnorm_backward(mk(0, 512, dt=HF), mk(0, 512, dt=HF), mk(512, dt=HF), rstd)
+    assert dw.shape == (512,) and not dw.any()
+
+
+def test_functions_take_other_widths_and_fp16(gpu_device):
+    """The autograd Functions and modules on a smaller model's shapes: hidden 1536 in fp16, head dim 64."""
+    from teletron_amd import fusedlayers as FL
+    d = O.make_adaln_inputs(2, 97, 1536, HF, seed=71)
+    want_out, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    x, sc, sh = (d[k].to(gpu_device).requires_grad_(True) for k in ("x", "scale", "shift"))
+    out = FL.AdaLNCustom(1536)(x, sc, sh)
+    out.backward(d["grad"].to(gpu_device))
+    fwd_16bit_ok(out.detach(), want_out, O.adaln_excuse(d["x"], d["scale"], d["shift"], want_out), "out")
+    grad_ok(x.grad, want_dx, "dx", allow=1e-4)
+    grad_ok(sc.grad, want_ds, "dscale")
+    grad_ok(sh.grad, want_dh, "dshift")
+    # QK-norm with head dim 64 on the transposed view: falls back to a contiguous copy, then any-width kernels
+    q = O.make_rmsnorm_inputs((2, 50, 6), 64, BF, seed=72)
+    want_q, want_dq, want_dw = O.eager_rmsnorm_fwd_bwd(q["x"].transpose(1, 2), q["weight"], q["grad"].transpose(1, 2))
+    xq = q["x"].to(gpu_device).requires_grad_(True)
+    wq = q["weight"].to(gpu_device).requires_grad_(True)
+    got = FL.RMSNormModelFunction.apply(xq.transpose(1, 2), wq, EPS, 64)
+    got.backward(q["grad"].to(gpu_device).transpose(1, 2))
+    fwd_16bit_ok(got.detach(), want_q, O.rmsnorm_excuse(want_q), "q")
+    assert xq.grad.shape == q["x"].shape
+    grad_ok(xq.grad.transpose(1, 2), want_dq, "dq")
+    grad_ok(wq.grad, want_dw, "dw")

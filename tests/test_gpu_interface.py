@@ -62,12 +62,16 @@ def test_adaln_function_value_errors(FL, gpu_device):
     x = torch.zeros(2, 4, 3072, dtype=torch.bfloat16, device=gpu_device)
     m = torch.zeros(2, 3072, dtype=torch.bfloat16, device=gpu_device)
     with pytest.raises(ValueError, match="cols"):
-        FL.AdaLNModelFunction.apply(x, m, m, EPS, 1024)
+        FL.AdaLNModelFunction.apply(x, m, m, EPS, 3076)          # rows are not whole 16-byte pieces
+    with pytest.raises(ValueError, match="not divisible"):
+        FL.AdaLNModelFunction.apply(x, m, m, EPS, 4000)
     with pytest.raises(ValueError, match="modulation rows"):
         FL.AdaLNModelFunction.apply(x, torch.zeros(4, 3072, dtype=torch.bfloat16, device=gpu_device),
                                     torch.zeros(4, 3072, dtype=torch.bfloat16, device=gpu_device), EPS, 3072)
-    with pytest.raises(ValueError):
+    with pytest.raises(ValueError, match="not divisible"):
         FL.RMSNormModelFunction.apply(x, torch.ones(3072, device=gpu_device), EPS, 1000)
+    with pytest.raises(ValueError, match="unsupported cols"):
+        FL.RMSNormModelFunction.apply(x.reshape(2, 1024, 12), torch.ones(12, device=gpu_device), EPS, 12)
 
 
 def test_rmsnorm_function_on_transposed_qk(FL, gpu_device):

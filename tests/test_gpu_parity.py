@@ -426,9 +426,9 @@ def test_error_statuses(capi, gpu_device):
     ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
     assert L.tt_rmsnorm_backward(vp(x), vp(w), vp(x), vp(x), vp(w), vp(r), 8, 3072, 0, vp(ws), need - 1, None) == 4
     assert L.tt_rmsnorm_backward(vp(x), vp(w), vp(x), vp(x), vp(w), vp(r), 8, 3072, 0, None, 0, None) == 4
-    with pytest.raises(capi.NormError):
-        capi.rmsnorm_forward(torch.zeros(4, 256, dtype=torch.bfloat16, device=gpu_device),
-                             torch.ones(256, dtype=torch.bfloat16, device=gpu_device), EPS)
+    with pytest.raises(capi.NormError):   # rows that are not whole 16-byte pieces
+        capi.rmsnorm_forward(torch.zeros(4, 260, dtype=torch.bfloat16, device=gpu_device),
+                             torch.ones(260, dtype=torch.bfloat16, device=gpu_device), EPS)
     torch.cuda.synchronize()
 
 

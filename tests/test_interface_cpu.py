@@ -31,15 +31,26 @@ def test_c_abi_exports_every_declared_symbol():
     assert L.tt_norm_status_string(0) == b"ok"
     assert L.tt_norm_status_string(4).startswith(b"workspace")
     assert L.tt_norm_supported(3072, capi.BF16) == 1 and L.tt_norm_supported(128, capi.F32) == 1
-    assert L.tt_norm_supported(1024, capi.BF16) == 0 and L.tt_norm_supported(3072, 5) == 0
+    assert L.tt_norm_supported(3072, 5) == 0
+    # every row of whole 16-byte pieces up to 1024 of them, in bf16 / fp16 / fp32
+    assert L.tt_norm_supported(1024, capi.BF16) == 1 and L.tt_norm_supported(8192, capi.F16) == 1
+    assert L.tt_norm_supported(4096, capi.F32) == 1 and L.tt_norm_supported(4100, capi.F32) == 0
+    assert L.tt_norm_supported(1000, capi.F32) == 1 and L.tt_norm_supported(1004, capi.BF16) == 0
+    assert L.tt_norm_supported(8200, capi.BF16) == 0
+    # the tuned shapes: the only ones the reference-contract, strided and gated entry points take
+    assert L.tt_norm_tuned(3072, capi.BF16) == 1 and L.tt_norm_tuned(128, capi.F32) == 1
+    assert L.tt_norm_tuned(3072, capi.F16) == 0 and L.tt_norm_tuned(256, capi.BF16) == 0
+    assert L.tt_rmsnorm_backward_from_out(None, None, None, None, None, None, 4, 256, 0, None, 0, None) == 2
+    assert L.tt_adaln_forward_xnorm(None, None, None, None, None, None, 1, 4, 3072, 1e-6, capi.F16, None) == 2
 
 
 def test_c_abi_argument_errors_need_no_gpu():
     from teletron_amd import capi
     L = capi.lib()
     assert L.tt_rmsnorm_forward(None, None, None, None, 4, 3072, 1e-6, 0, None) == 1      # null pointers
-    assert L.tt_rmsnorm_forward(None, None, None, None, 4, 1000, 1e-6, 0, None) == 2      # unsupported cols
-    assert b"cols=1000" in L.tt_norm_last_error()
+    assert L.tt_rmsnorm_forward(None, None, None, None, 4, 1004, 1e-6, 0, None) == 2      # unsupported cols
+    assert b"cols=1004" in L.tt_norm_last_error()
+    assert L.tt_rmsnorm_forward(None, None, None, None, 4, 1000, 1e-6, 0, None) == 1      # supported; null pointers
     assert L.tt_adaln_forward(None, None, None, None, None, None, 0, 4, 3072, 1e-6, 0, None) == 1
     assert L.tt_norm_stream_copy(None, None, 32, None) == 1
 
@@ -104,8 +115,11 @@ def test_rmsnorm_module_env_gate_and_eager_branch(monkeypatch):
     assert FL.fused_kernels_requested()
     with pytest.raises(ValueError, match="GPU tensor"):   # fused requested: no quiet CPU fallback
         m(d["x"])
-    other = RMSNorm(96, config=None)                        # a width the kernels are not built for
-    assert other(torch.ones(2, 96)).shape == (2, 96)
+    other = RMSNorm(98, config=None)                        # a width the kernels are not built for
+    assert other(torch.ones(2, 98)).shape == (2, 98)        # (rows must be whole 16-byte pieces): eager
+    assert FL.cols_supported(96, torch.float32) and FL.cols_supported(96, torch.float16)
+    assert not FL.cols_supported(100, torch.bfloat16) and not FL.cols_supported(8200, torch.bfloat16)
+    assert not FL.cols_supported(128, torch.float64)
 
 
 def test_adaln_zero_modules_eager_branch_matches_oracle():
@@ -128,8 +142,11 @@ def test_adaln_zero_modules_eager_branch_matches_oracle():
     assert torch.equal(gate3, c3[2])
     with pytest.raises(ValueError, match="norm_type"):
         FL.FusedAdaLayerNormZeroSingle(C, linear_parallel=False, norm_type="nope")
-    with pytest.raises(ValueError, match="embedding_dim"):
-        FL.FusedAdaLayerNormZero(C, linear_parallel=False, fused_kernels=True)
+    with pytest.raises(ValueError, match="unsupported cols 66"):   # not whole 16-byte pieces
+        FL.FusedAdaLayerNormZero(66, linear_parallel=False, fused_kernels=True)
+    fused = FL.FusedAdaLayerNormZero(C, linear_parallel=False, fused_kernels=True)   # 64 columns: any-width kernels
+    with pytest.raises(ValueError, match="GPU tensor"):                               # and no quiet CPU fallback
+        fused(x, emb=temb)
 
 
 def test_fp32_layer_norm():
