@@ -30,18 +30,18 @@ HBM_PEAK_GBS = 8000.0
 # (scaled by the same counters on the plain copy kernel); None until measured.
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE KiB * 2.000 + WRITE_SIZE KiB * 1.000) * 1024, see profiles/bench_cfg4_all_kernels.md
-    "rmsnorm_backward": int((714785.3 * 2.0 + 715874.1) * 1024),
-    "adaln_backward": int((716635.2 * 2.0 + 718944.0) * 1024),
-    "rmsnorm_forward": int((356450.6 * 2.0 + 713737.9) * 1024),
-    "adaln_forward": int((356497.1 * 2.0 + 714656.4) * 1024),
+    "rmsnorm_backward": int((714789.7 * 2.0 + 715874.8) * 1024),
+    "adaln_backward": int((716633.5 * 2.0 + 718944.0) * 1024),
+    "rmsnorm_forward": int((356450.6 * 2.0 + 713734.8) * 1024),
+    "adaln_forward": int((356500.1 * 2.0 + 714670.7) * 1024),
 }
 
 
 KERNEL_SYMBOL = {
     "rmsnorm_forward": "ttn::rmsnorm_fwd_kernel<ttn::bf16_t, 3072, ttn::DenseRows>",
     "rmsnorm_backward": "ttn::rmsnorm_bwd_kernel<ttn::bf16_t, 3072, false, ttn::DenseRows>",
-    "adaln_forward": "ttn::adaln_fwd_kernel<ttn::bf16_t, 3072, false>",
-    "adaln_backward": "ttn::adaln_bwd_kernel<ttn::bf16_t, 3072, false>",
+    "adaln_forward": "ttn::adaln_fwd_kernel<ttn::bf16_t, 3072, false, false>",
+    "adaln_backward": "ttn::adaln_bwd_kernel<ttn::bf16_t, 3072, false, false>",
 }
 
 

@@ -24,7 +24,7 @@ struct PadGeom {
     static constexpr int LANES = LANES_;
     static constexpr int CHUNKS = CHUNKS_;
     static constexpr int RPW = kWaveSize / LANES;
-    static_assert(LANES == 16 || LANES == 32 || LANES == 64, "row must fill whole DPP rows");
+    static_assert(LANES == 8 || LANES == 16 || LANES == 32 || LANES == 64, "row must fill an aligned lane group");
     static_assert(LANES == 64 || CHUNKS == 1, "only full wavefronts take several accesses per lane");
 };
 
@@ -471,6 +471,7 @@ struct GeomChoice {
     int lanes, chunks;
 };
 static GeomChoice choose_geometry(int pieces) {
+    if (pieces <= 8) return {8, 1};
     if (pieces <= 16) return {16, 1};
     if (pieces <= 32) return {32, 1};
     const int need = (pieces + 63) / 64;
@@ -481,7 +482,7 @@ static GeomChoice choose_geometry(int pieces) {
 
 // Calls F<T, LANES, CHUNKS>::run(args...) for the run-time (dtype, geometry).
 #define TTN_ANYWIDTH_GEOMS(X, T) \
-    X(T, 16, 1) X(T, 32, 1) X(T, 64, 1) X(T, 64, 2) X(T, 64, 3) X(T, 64, 4) X(T, 64, 6) X(T, 64, 8) X(T, 64, 12) X(T, 64, 16)
+    X(T, 8, 1) X(T, 16, 1) X(T, 32, 1) X(T, 64, 1) X(T, 64, 2) X(T, 64, 3) X(T, 64, 4) X(T, 64, 6) X(T, 64, 8) X(T, 64, 12) X(T, 64, 16)
 
 template <template <typename, int, int> class F, typename... Args>
 static int dispatch(int dtype, GeomChoice gc, Args... args) {

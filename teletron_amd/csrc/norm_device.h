@@ -191,12 +191,21 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// Sum over each aligned group of LANES lanes (16, 32 or 64); every lane of the
+// Sum over each aligned group of 8 lanes; every lane gets its group's sum.
+__device__ __forceinline__ float row8_sum(float v) {
+    v += dpp_take<kDppQuadXor1, 0xf>(v);
+    v += dpp_take<kDppQuadXor2, 0xf>(v);
+    v += dpp_take<kDppRowHalfMirror, 0xf>(v);
+    return v;
+}
+
+// Sum over each aligned group of LANES lanes (8, 16, 32 or 64); every lane of the
 // group gets the sum.  The 64-lane form funnels the four DPP-row sums into
 // lane 63 with two row broadcasts and returns it through a scalar register,
 // so it costs no LDS traffic at all.
 template <int LANES>
 __device__ __forceinline__ float group_sum(float v) {
+    if constexpr (LANES == 8) return row8_sum(v);
     v = row16_sum(v);
     if constexpr (LANES == 32) {
         v += __shfl_xor(v, 16, kWaveSize);
@@ -214,6 +223,7 @@ template <int LANES>
 __device__ __forceinline__ float fold_rows_of_wave(float v) {
     if constexpr (LANES <= 32) v += __shfl_xor(v, 32, kWaveSize);
     if constexpr (LANES <= 16) v += __shfl_xor(v, 16, kWaveSize);
+    if constexpr (LANES <= 8) v += __shfl_xor(v, 8, kWaveSize);
     return v;
 }
 

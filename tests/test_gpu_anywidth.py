@@ -11,16 +11,16 @@ pytestmark = pytest.mark.gpu
 EPS = 1e-6
 
 BF, HF, F32 = torch.bfloat16, torch.float16, torch.float32
-# (cols, rows, dtype): every kernel geometry (16 / 32 lanes; 1, 2, 3, 4, 6, 8, 12, 16 accesses per lane),
+# (cols, rows, dtype): every kernel geometry (8 / 16 / 32 lanes; 1, 2, 3, 4, 6, 8, 12, 16 accesses per lane),
 # full and ragged last accesses, row counts that do not fill the last wavefront
 RMS_CASES = [
-    (8, 5, BF), (64, 1001, BF), (96, 130, BF), (128, 77, HF), (200, 513, BF), (256, 4099, BF), (512, 300, BF),
+    (8, 5, BF), (40, 300, HF), (64, 1001, BF), (96, 130, BF), (128, 77, HF), (200, 513, BF), (256, 4099, BF), (512, 300, BF),
     (768, 257, BF), (1000, 50, BF), (1024, 1000, BF), (1536, 333, HF), (2048, 77, BF), (2560, 65, BF),
     (3072, 300, HF), (3080, 33, BF), (4096, 129, BF), (5120, 130, BF), (6144, 70, HF), (8192, 66, BF),
     (8192, 9, HF), (4, 3, F32), (64, 100, F32), (256, 1000, F32), (1000, 77, F32), (2048, 129, F32), (4096, 40, F32),
 ]
 ADALN_CASES = [
-    (1, 5, 8, BF), (3, 333, 64, BF), (2, 65, 96, HF), (2, 1001, 256, BF), (4, 100, 512, BF), (1, 257, 1000, BF),
+    (1, 5, 8, BF), (2, 301, 56, HF), (3, 333, 64, BF), (2, 65, 96, HF), (2, 1001, 256, BF), (4, 100, 512, BF), (1, 257, 1000, BF),
     (2, 130, 1024, HF), (3, 77, 1536, BF), (2, 300, 2048, BF), (5, 33, 3072, HF), (2, 65, 4096, BF),
     (2, 130, 5120, BF), (3, 40, 6144, BF), (2, 35, 6144, HF), (2, 66, 8192, BF), (1, 9, 8192, HF),
     (2, 50, 64, F32), (3, 100, 1000, F32), (2, 40, 4096, F32),
