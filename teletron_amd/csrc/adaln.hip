@@ -22,8 +22,13 @@
 #ifndef TTN_ADALN_BWD_ROW_BUFFERS
 #define TTN_ADALN_BWD_ROW_BUFFERS 1
 #endif
-#ifndef TTN_GATED_LATE_OPERANDS  // gated backward, 2-byte rows: fetch attn and e in the second pass
-#define TTN_GATED_LATE_OPERANDS 0
+// Gated backward, 2-byte rows: when attn and e (the gradient arriving at h2) are fetched.
+//   0: with g and x, one row at a time
+//   1: at the start of a row's processing (they are needed in its second pass only), while g and x of
+//      the NEXT row are requested between the two passes (two g/x buffers)
+//   2: in the second pass, where they are used
+#ifndef TTN_GATED_OPERANDS
+#define TTN_GATED_OPERANDS 1
 #endif
 #ifndef TTN_ADALN_BWD_PREFETCH_MID
 #define TTN_ADALN_BWD_PREFETCH_MID 0
@@ -242,7 +247,8 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     // gate[sample]: unpacked once for 2-byte elements; 4-byte rows have no registers to spare and
     // re-read it (cache hits) where it is used
     constexpr bool kGateResident = GATED && sizeof(T) == 2;
-    constexpr bool kEarlyOperands = kGateResident && !TTN_GATED_LATE_OPERANDS;  // attn, e fetched with g, x
+    constexpr bool kEarlyOperands = kGateResident && TTN_GATED_OPERANDS == 0;    // attn, e fetched with g, x
+    constexpr bool kStartOperands = kGateResident && TTN_GATED_OPERANDS == 1;    // ... when processing starts
     [[maybe_unused]] float gatev[kGateResident ? CHUNKS : 1][VEC];
     if constexpr (kGateResident) {
 #pragma unroll
@@ -298,6 +304,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     auto process = [&](const RowRegs &b, auto &&between_passes) {
         const float r = b.r, mu = b.mu;
         const float nmr = -(mu * r);  // xhat = x*r + nmr
+        [[maybe_unused]] u32x4 ar[kStartOperands ? CHUNKS : 1], er[kStartOperands ? CHUNKS : 1];
+        if constexpr (kStartOperands) {
+            const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + b.row * C) + l;
+            const u32x4 *pe = reinterpret_cast<const u32x4 *>(e + b.row * C) + l;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) ar[k] = b.ok ? load16_stream(pa + k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k)
+                er[k] = (b.ok && e != nullptr) ? load16_stream(pe + k * LANES) : u32x4{0, 0, 0, 0};
+        }
         // pass 1: gx = rnd(g*t) kept packed; s1 = sum_c gx; s2 = sum_c gx * xhat
         u32x4 gxp[CHUNKS];
         float s1 = 0.0f, s2 = 0.0f;
@@ -355,6 +371,9 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 if constexpr (kEarlyOperands) {
                     E::unpack(b.e[k], ev);
                     E::unpack(b.a[k], av);
+                } else if constexpr (kStartOperands) {
+                    E::unpack(er[k], ev);
+                    E::unpack(ar[k], av);
                 } else {
                     const int64_t at = b.row * (C / VEC) + l + k * LANES;
                     const u32x4 zero{0, 0, 0, 0};
@@ -395,7 +414,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
     int64_t grp = (int64_t)slot * kRowWaves + wave;
-    row_pipeline<kRowBuffers, TTN_ADALN_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
+    if constexpr (kStartOperands)
+        row_pipeline<2, true, RowRegs>(grp, groups, stride, fetch, process);
+    else
+        row_pipeline<kRowBuffers, TTN_ADALN_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
     flush_column_partials<G, NSETS>(acc, partial + (int64_t)blockIdx.x * (NSETS * C), lds);
 }
 
