@@ -10,6 +10,9 @@ call measured with HIP events, and the reference's eager path timed on the
 host CPU on a bounded sample of the same workload.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+`--workload` selects one of the other configurations (cfg1, cfg2, cfg2-strided, cfg3, cfg5) or
+the gated residual + AdaLN call site instead; same timing method, same JSON line, no CPU leg.
 """
 import argparse
 import ctypes
@@ -45,12 +48,147 @@ KERNEL_SYMBOL = {
 }
 
 
+WORKLOADS = {
+    "cfg4": "cfg4: 118800 tokens x 3072 bf16; fused RMSNorm(3072) fwd+bwd + fused AdaLN fwd+bwd "
+            "per step (4 C-ABI calls), eps 1e-6, one modulation row",
+    "cfg1": "cfg1: 8192 x 3072 fp32; fused RMSNorm fwd+bwd (2 C-ABI calls)",
+    "cfg2": "cfg2: q and k of one CP=4 rank, [1, 29700, 24, 128] bf16 each, contiguous; per-head RMSNorm(128) "
+            "fwd+bwd on both (4 C-ABI calls)",
+    "cfg2-strided": "cfg2 on the call site's own layout: q and k are transposed [B, H, S, D] views into the fused "
+                    "[1, 29700, 24, 384] QKV projection, read in place; outputs and dx contiguous (4 C-ABI calls)",
+    "cfg3": "cfg3: 29700 tokens x 3072 bf16; fused AdaLN fwd+bwd (2 C-ABI calls)",
+    "cfg5": "cfg5: batch 4 x 11056 tokens x 3072 bf16, one modulation row per sample; AdaLN then RMSNorm(3072), "
+            "forward and backward of the chain (4 C-ABI calls)",
+    "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
+             "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
+}
+
+
+def build_workload(name, torch, capi, dev):
+    """Allocates the inputs of one workload in HBM and returns (calls, tensor_bytes, tokens_per_step, dtype)
+    with calls = [(call name, closure, algorithmic traffic in tensors)]."""
+    L = capi.lib()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def ck(st, what):
+        if st != 0:
+            raise RuntimeError(f"{what}: {L.tt_norm_last_error().decode()}")
+
+    def rnd(*shape, dtype, k=1.0, bias=0.0):
+        return (bias + k * torch.randn(*shape, device=dev, generator=gen)).to(dtype)
+
+    f32 = lambda n: torch.empty(n, device=dev, dtype=torch.float32)
+    scratch = lambda n: torch.empty(max(int(n), 16), device=dev, dtype=torch.uint8)
+
+    def rms_pair(x, grad, w, tag=""):
+        rows, cols = x.numel() // x.shape[-1], x.shape[-1]
+        dt = capi._DTYPES[x.dtype]
+        out, dx, rstd, dw = torch.empty_like(x), torch.empty_like(x), f32(rows), torch.empty_like(w)
+        n = L.tt_rmsnorm_backward_workspace_bytes(rows, cols, dt)
+        ws = scratch(n)
+        fwd = lambda: ck(L.tt_rmsnorm_forward(p(out), p(rstd), p(x), p(w), rows, cols, EPS, dt, stream), "rms fwd")
+        bwd = lambda: ck(L.tt_rmsnorm_backward(p(dx), p(dw), p(grad), p(x), p(w), p(rstd), rows, cols, dt, p(ws), n,
+                                               stream), "rms bwd")
+        return [("rmsnorm_forward" + tag, fwd, 2), ("rmsnorm_backward" + tag, bwd, 3)], out
+
+    def adaln_pair(x, grad, scale, shift):
+        batch, cols = scale.shape
+        rps = x.numel() // cols // batch
+        dt = capi._DTYPES[x.dtype]
+        out, dx = torch.empty_like(x), torch.empty_like(x)
+        mean, rstd = f32(batch * rps), f32(batch * rps)
+        dsc, dsh = torch.empty_like(scale), torch.empty_like(scale)
+        n = L.tt_adaln_backward_workspace_bytes(batch, rps, cols, dt)
+        ws = scratch(n)
+        fwd = lambda: ck(L.tt_adaln_forward(p(out), p(mean), p(rstd), p(x), p(scale), p(shift), batch, rps, cols,
+                                            EPS, dt, stream), "adaln fwd")
+        bwd = lambda: ck(L.tt_adaln_backward(p(dx), p(dsc), p(dsh), p(grad), p(x), p(scale), p(mean), p(rstd), batch,
+                                             rps, cols, dt, p(ws), n, stream), "adaln bwd")
+        return [("adaln_forward", fwd, 2), ("adaln_backward", bwd, 3)], out
+
+    bf = torch.bfloat16
+    if name in ("cfg4", "cfg3"):
+        rows = ROWS if name == "cfg4" else 29700
+        x, grad = rnd(rows, COLS, dtype=bf), rnd(rows, COLS, dtype=bf)
+        scale, shift = rnd(1, COLS, dtype=bf, k=0.1), rnd(1, COLS, dtype=bf, k=0.1)
+        calls = []
+        if name == "cfg4":
+            calls += rms_pair(x, grad, rnd(COLS, dtype=bf, k=0.02, bias=1.0))[0]
+        calls += adaln_pair(x, grad, scale, shift)[0]
+        return calls, rows * COLS * 2, rows * (2 if name == "cfg4" else 1), "bf16", x
+    if name == "cfg1":
+        x, grad = rnd(8192, COLS, dtype=torch.float32), rnd(8192, COLS, dtype=torch.float32)
+        calls, _ = rms_pair(x, grad, rnd(COLS, dtype=torch.float32, k=0.02, bias=1.0))
+        return calls, 8192 * COLS * 4, 8192, "f32", x
+    if name == "cfg2":
+        calls = []
+        for tag in ("_q", "_k"):
+            x, grad = rnd(712800, 128, dtype=bf), rnd(712800, 128, dtype=bf)
+            calls += rms_pair(x, grad, rnd(128, dtype=bf, k=0.02, bias=1.0), tag)[0]
+        return calls, 712800 * 128 * 2, 29700, "bf16", x
+    if name == "cfg2-strided":
+        B, S, H, D = 1, 29700, 24, 128
+        mixed = rnd(B, S, H, 3 * D, dtype=bf)
+        calls = []
+        for i, tag in enumerate(("_q", "_k")):
+            view = mixed[..., i * D:(i + 1) * D].transpose(1, 2)          # [B, H, S, D], strides (S*H*3D, 3D, H*3D, 1)
+            grad = rnd(B, H, S, D, dtype=bf)
+            w = rnd(D, dtype=bf, k=0.02, bias=1.0)
+            out, dx, rstd, dw = torch.empty_like(grad), torch.empty_like(grad), f32(B * H * S), torch.empty_like(w)
+            xs, ds = view.stride(), dx.stride()
+            n = L.tt_rmsnorm_backward_workspace_bytes(B * H * S, D, capi.BF16)
+            ws = scratch(n)
+            fwd = (lambda out=out, rstd=rstd, view=view, w=w, xs=xs:
+                   ck(L.tt_rmsnorm_forward_strided(p(out), p(rstd), p(view), p(w), B, H, S, xs[0], xs[1], xs[2], D,
+                                                   EPS, capi.BF16, stream), "rms fwd strided"))
+            bwd = (lambda dx=dx, dw=dw, grad=grad, view=view, w=w, rstd=rstd, xs=xs, ds=ds, ws=ws, n=n:
+                   ck(L.tt_rmsnorm_backward_strided(p(dx), p(dw), p(grad), p(view), p(w), p(rstd), B, H, S, xs[0],
+                                                    xs[1], xs[2], ds[0], ds[1], ds[2], D, capi.BF16, p(ws), n,
+                                                    stream), "rms bwd strided"))
+            calls += [("rmsnorm_forward_strided" + tag, fwd, 2), ("rmsnorm_backward_strided" + tag, bwd, 3)]
+        return calls, B * H * S * D * 2, S, "bf16", mixed
+    if name == "cfg5":
+        B, S = 4, 11056
+        x, grad = rnd(B, S, COLS, dtype=bf, k=2.0), rnd(B, S, COLS, dtype=bf)
+        scale, shift = rnd(B, COLS, dtype=bf, k=0.1), rnd(B, COLS, dtype=bf, k=0.1)
+        ada, y = adaln_pair(x, grad, scale, shift)
+        ada[0][1]()                                                         # y = AdaLN(x) feeds the RMSNorm
+        rms, _ = rms_pair(y, grad, rnd(COLS, dtype=bf, k=0.02, bias=1.0))
+        # chain order: AdaLN fwd, RMSNorm fwd, RMSNorm bwd, AdaLN bwd (the gradient buffers are stand-ins of the
+        # right size: timing does not depend on their values)
+        return [ada[0], rms[0], rms[1], ada[1]], B * S * COLS * 2, B * S, "bf16", x
+    if name == "gated":
+        B, S = 1, ROWS
+        h, a = rnd(B, S, COLS, dtype=bf), rnd(B, S, COLS, dtype=bf)
+        go, g2 = rnd(B, S, COLS, dtype=bf, k=0.1), rnd(B, S, COLS, dtype=bf, k=0.1)
+        gate, scale, shift = (rnd(B, COLS, dtype=bf, k=0.3) for _ in range(3))
+        h2, out, dh, da = (torch.empty_like(h) for _ in range(4))
+        mean, rstd = f32(B * S), f32(B * S)
+        dq, dsc, dsh = (torch.empty_like(gate) for _ in range(3))
+        n = L.tt_gated_residual_adaln_backward_workspace_bytes(B, S, COLS, capi.BF16)
+        ws = scratch(n)
+        fwd = lambda: ck(L.tt_gated_residual_adaln_forward(p(h2), p(out), p(mean), p(rstd), p(h), p(a), p(gate),
+                                                           p(scale), p(shift), B, S, COLS, EPS, capi.BF16, stream),
+                         "gated fwd")
+        bwd = lambda: ck(L.tt_gated_residual_adaln_backward(p(dh), p(da), p(dq), p(dsc), p(dsh), p(go), p(g2), p(h2),
+                                                            p(a), p(gate), p(scale), p(mean), p(rstd), B, S, COLS,
+                                                            capi.BF16, p(ws), n, stream), "gated bwd")
+        return [("gated_residual_adaln_forward", fwd, 4), ("gated_residual_adaln_backward", bwd, 6)], \
+            S * COLS * 2, S, "bf16", h
+    raise ValueError(name)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU eager timing")
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS),
+                    help="cfg4 (default) is the headline step; the others measure the remaining "
+                         "configurations and the call sites around the path with the same method")
     return ap.parse_args()
 
 
@@ -100,50 +238,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L = capi.lib()
-    bf = torch.bfloat16
-
-    gen = torch.Generator(device=dev).manual_seed(0)
-    x = torch.randn(ROWS, COLS, device=dev, generator=gen).to(bf)
-    grad = torch.randn(ROWS, COLS, device=dev, generator=gen).to(bf)
-    weight = (1 + 0.02 * torch.randn(COLS, device=dev, generator=gen)).to(bf)
-    scale = (0.1 * torch.randn(1, COLS, device=dev, generator=gen)).to(bf)
-    shift = (0.1 * torch.randn(1, COLS, device=dev, generator=gen)).to(bf)
-    out = torch.empty_like(x)
-    dx = torch.empty_like(x)
-    rstd = torch.empty(ROWS, device=dev, dtype=torch.float32)
-    mean = torch.empty(ROWS, device=dev, dtype=torch.float32)
-    dweight = torch.empty_like(weight)
-    dscale = torch.empty_like(scale)
-    dshift = torch.empty_like(scale)
-    ws_rms_n = L.tt_rmsnorm_backward_workspace_bytes(ROWS, COLS, capi.BF16)
-    ws_ada_n = L.tt_adaln_backward_workspace_bytes(1, ROWS, COLS, capi.BF16)
-    ws = torch.empty(max(ws_rms_n, ws_ada_n), device=dev, dtype=torch.uint8)
-
-    p = lambda t: ctypes.c_void_p(t.data_ptr())
-    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-
-    def ck(st, what):
-        if st != 0:
-            raise RuntimeError(f"{what}: {L.tt_norm_last_error().decode()}")
-
-    def rms_fwd():
-        ck(L.tt_rmsnorm_forward(p(out), p(rstd), p(x), p(weight), ROWS, COLS, EPS, capi.BF16, stream), "rms fwd")
-
-    def rms_bwd():
-        ck(L.tt_rmsnorm_backward(p(dx), p(dweight), p(grad), p(x), p(weight), p(rstd), ROWS, COLS, capi.BF16,
-                                 p(ws), ws_rms_n, stream), "rms bwd")
-
-    def ada_fwd():
-        ck(L.tt_adaln_forward(p(out), p(mean), p(rstd), p(x), p(scale), p(shift), 1, ROWS, COLS, EPS, capi.BF16,
-                              stream), "adaln fwd")
-
-    def ada_bwd():
-        ck(L.tt_adaln_backward(p(dx), p(dscale), p(dshift), p(grad), p(x), p(scale), p(mean), p(rstd), 1, ROWS,
-                               COLS, capi.BF16, p(ws), ws_ada_n, stream), "adaln bwd")
-
-    calls = [("rmsnorm_forward", rms_fwd, 2), ("rmsnorm_backward", rms_bwd, 3),
-             ("adaln_forward", ada_fwd, 2), ("adaln_backward", ada_bwd, 3)]
-    tensor_bytes = ROWS * COLS * 2
+    calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)
+    headline = args.workload == "cfg4"
 
     names = [n for n, _, _ in calls]
     mults = dict((n, m) for n, _, m in calls)
@@ -218,20 +314,23 @@ def main():
     dom_ms /= args.steps
     achieved = mults[dom] * tensor_bytes / (dom_ms * 1e-3) / 1e9
 
-    # streaming-copy yardstick (read N*C*2, write N*C*2) with the same access pattern
+    # streaming-copy yardstick (read one tensor, write one tensor) with the same access pattern
+    src = a_tensor.reshape(-1)[:tensor_bytes // a_tensor.element_size()]
+    dst = torch.empty_like(src)
     for _ in range(3):
-        capi.stream_copy(out, x)
+        capi.stream_copy(dst, src)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(10):
-        capi.stream_copy(out, x)
+        capi.stream_copy(dst, src)
     e1.record()
     torch.cuda.synchronize()
     copy_gbs = 2 * tensor_bytes / (e0.elapsed_time(e1) / 10) / 1e6
 
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     result = {
-        "metric": "fwd+bwd HBM GB/s and % of peak for RMSNorm/AdaLN at 118800x3072 bf16",
+        "metric": "fwd+bwd HBM GB/s and % of peak for RMSNorm/AdaLN at 118800x3072 bf16" if headline
+                  else "fwd+bwd HBM GB/s and % of peak, workload " + args.workload,
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -241,22 +340,23 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": dtype_name,
         "data": "synthetic",
-        "config": {"workload": "cfg4: 118800 tokens x 3072 bf16; fused RMSNorm(3072) fwd+bwd + fused AdaLN fwd+bwd "
-                               "per step (4 C-ABI calls), eps 1e-6, one modulation row",
-                   "rows": ROWS, "cols": COLS, "algorithmic_bytes_per_step": step_bytes},
+        "config": {"workload": WORKLOADS[args.workload], "tensor_bytes": tensor_bytes,
+                   "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "tokens_per_s": round(2 * ROWS / (ms_per_step * 1e-3), 1),
+        "tokens_per_s": round(tokens_per_step / (ms_per_step * 1e-3), 1),
         "per_call_untimed": per_call,
         "stream_copy_GB/s": round(copy_gbs, 1),
-        "roofline": {"bound": "hbm", "kernel": KERNEL_SYMBOL[dom], "call": "tt_" + dom,
+        "roofline": {"bound": "hbm", "kernel": KERNEL_SYMBOL.get(dom) if headline else None, "call": "tt_" + dom.removesuffix("_q").removesuffix("_k"),
                      "avg_us": round(dom_ms * 1e3, 1),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom)},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if headline else None},
     }
-    if not args.no_cpu_baseline:
+    if headline:
+        result["config"].update({"rows": ROWS, "cols": COLS})
+    if headline and not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_eager_baseline()
     print(json.dumps(result))
 
