@@ -5,7 +5,7 @@ The reference repository holds no vectors for this path and its Python module
 cannot be imported here (its top-level imports need diffusers and megatron),
 so these vectors come from the restatement, whose arithmetic is pinned by the
 checks in tests/test_oracle.py.  bf16 tensors are stored as their uint16 bit
-patterns.  Run from the repo root:  python tests/golden/make_golden.py
+patterns, fp16 tensors as numpy float16.  Run from the repo root:  python tests/golden/make_golden.py
 """
 import os
 import sys
@@ -26,6 +26,12 @@ CASES = {
     "adaln_bf16_b1": ("adaln", dict(batch=1, seq=9, cols=3072, dtype=torch.bfloat16, seed=15)),
     "adaln_bf16_b3": ("adaln", dict(batch=3, seq=5, cols=3072, dtype=torch.bfloat16, seed=16, sigma=2.0)),
     "adaln_f32_b2": ("adaln", dict(batch=2, seq=4, cols=3072, dtype=torch.float32, seed=17)),
+    # other widths and fp16 (the any-width kernels)
+    "rms_f16_c1000": ("rmsnorm", dict(lead_shape=(6,), cols=1000, dtype=torch.float16, seed=18)),
+    "rms_bf16_c5120": ("rmsnorm", dict(lead_shape=(3,), cols=5120, dtype=torch.bfloat16, seed=19)),
+    "adaln_f16_c64": ("adaln", dict(batch=2, seq=9, cols=64, dtype=torch.float16, seed=20)),
+    # gated residual update + AdaLN, with a gradient arriving at h2
+    "gated_bf16_b2": ("gated", dict(batch=2, seq=4, cols=3072, dtype=torch.bfloat16, seed=21)),
 }
 
 
@@ -44,13 +50,19 @@ def main():
             d = O.make_rmsnorm_inputs(**kw)
             out, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
             res = {"out": out, "dx": dx, "dweight": dw}
-        else:
+        elif op == "adaln":
             d = O.make_adaln_inputs(**kw)
             out, dx, ds, dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
             res = {"out": out, "dx": dx, "dscale": ds, "dshift": dh}
+        else:
+            names = ("h", "attn", "gate", "scale", "shift", "grad", "grad_h2")
+            d = dict(zip(names, O.make_gated_inputs(**kw)))
+            got = O.eager_gated_residual_adaln_fwd_bwd(d["h"], d["attn"], d["gate"], d["scale"], d["shift"],
+                                                       d["grad"], d["grad_h2"])
+            res = dict(zip(("h2", "out", "dh", "dattn", "dgate", "dscale", "dshift"), got))
         for k, v in {**d, **res}.items():
             blob[f"{name}/{k}"] = to_np(v)
-        blob[f"{name}/is_bf16"] = np.array(kw["dtype"] == torch.bfloat16)
+        blob[f"{name}/is_16bit"] = np.array(kw["dtype"] != torch.float32)
     np.savez_compressed(os.path.join(HERE, "norm_golden.npz"), **blob)
     print("wrote", len(blob), "arrays")
 

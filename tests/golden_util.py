@@ -1,4 +1,4 @@
-"""Loader for tests/golden/norm_golden.npz (bf16 stored as uint16 bit patterns)."""
+"""Loader for tests/golden/norm_golden.npz (bf16 stored as uint16 bit patterns, fp16 as float16)."""
 import os
 
 import numpy as np
@@ -15,13 +15,13 @@ def load_golden():
         cases.setdefault(name, {})[field] = z[key]
     out = {}
     for name, fields in cases.items():
-        is_bf16 = bool(fields.pop("is_bf16"))
+        is_16bit = bool(fields.pop("is_16bit"))
         d = {}
         for k, a in fields.items():
             if a.dtype == np.uint16:
                 d[k] = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
             else:
                 d[k] = torch.from_numpy(a.copy())
-        d["is_bf16"] = is_bf16
+        d["is_16bit"] = is_16bit
         out[name] = d
     return out

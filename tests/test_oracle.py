@@ -372,16 +372,20 @@ def test_staged_rounding_points_hold_for_fp16_and_other_widths(cols):
 
 def test_golden_vectors_reproduce():
     gold = load_golden()
-    assert len(gold) == 7
+    assert len(gold) == 11
     for name, d in gold.items():
         if name.startswith("rms"):
             out, dx, dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
             got = {"out": out, "dx": dx, "dweight": dw}
-        else:
+        elif name.startswith("adaln"):
             out, dx, ds, dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
             got = {"out": out, "dx": dx, "dscale": ds, "dshift": dh}
+        else:
+            res = O.eager_gated_residual_adaln_fwd_bwd(d["h"], d["attn"], d["gate"], d["scale"], d["shift"],
+                                                       d["grad"], d["grad_h2"])
+            got = dict(zip(("h2", "out", "dh", "dattn", "dgate", "dscale", "dshift"), res))
         for k, v in got.items():
-            if d["is_bf16"]:
+            if d["is_16bit"]:
                 # thread count may change a summation order: allow 1 ulp on a handful of elements
                 rep = O.compare_bf16_ulp(v, d[k])
                 assert rep.frac_exact > 0.995 and O.frac_outside(v, d[k], 1e-2, 1e-3) == 0.0, (name, k, rep)
