@@ -59,6 +59,8 @@ WORKLOADS = {
     "cfg3": "cfg3: 29700 tokens x 3072 bf16; fused AdaLN fwd+bwd (2 C-ABI calls)",
     "cfg5": "cfg5: batch 4 x 11056 tokens x 3072 bf16, one modulation row per sample; AdaLN then RMSNorm(3072), "
             "forward and backward of the chain (4 C-ABI calls)",
+    "w1536-f16": "237600 tokens x 1536 fp16 (a smaller model's hidden size, the any-width kernels); fused RMSNorm "
+                 "fwd+bwd + fused AdaLN fwd+bwd per step (4 C-ABI calls)",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -109,15 +111,16 @@ def build_workload(name, torch, capi, dev):
         return [("adaln_forward", fwd, 2), ("adaln_backward", bwd, 3)], out
 
     bf = torch.bfloat16
-    if name in ("cfg4", "cfg3"):
-        rows = ROWS if name == "cfg4" else 29700
-        x, grad = rnd(rows, COLS, dtype=bf), rnd(rows, COLS, dtype=bf)
-        scale, shift = rnd(1, COLS, dtype=bf, k=0.1), rnd(1, COLS, dtype=bf, k=0.1)
+    if name in ("cfg4", "cfg3", "w1536-f16"):
+        rows, cols, dt = {"cfg4": (ROWS, COLS, bf), "cfg3": (29700, COLS, bf),
+                          "w1536-f16": (2 * ROWS, 1536, torch.float16)}[name]
+        x, grad = rnd(rows, cols, dtype=dt), rnd(rows, cols, dtype=dt)
+        scale, shift = rnd(1, cols, dtype=dt, k=0.1), rnd(1, cols, dtype=dt, k=0.1)
         calls = []
-        if name == "cfg4":
-            calls += rms_pair(x, grad, rnd(COLS, dtype=bf, k=0.02, bias=1.0))[0]
+        if name != "cfg3":
+            calls += rms_pair(x, grad, rnd(cols, dtype=dt, k=0.02, bias=1.0))[0]
         calls += adaln_pair(x, grad, scale, shift)[0]
-        return calls, rows * COLS * 2, rows * (2 if name == "cfg4" else 1), "bf16", x
+        return calls, rows * cols * 2, rows * (1 if name == "cfg3" else 2), "f16" if dt != bf else "bf16", x
     if name == "cfg1":
         x, grad = rnd(8192, COLS, dtype=torch.float32), rnd(8192, COLS, dtype=torch.float32)
         calls, _ = rms_pair(x, grad, rnd(COLS, dtype=torch.float32, k=0.02, bias=1.0))
