@@ -14,7 +14,11 @@ What differs from the reference, on purpose:
   * scale/shift may carry one row per sample ([B, C]) and their gradients come
     back per sample, which is what the eager formula at :223 computes; the
     reference kernels only handle a single modulation row;
-  * both operators accept 128 and 3072 columns, bf16 and fp32;
+  * both operators accept any row of whole 16-byte pieces (up to 8192 two-byte or
+    4096 four-byte columns) in bf16, fp16 or fp32; 128 and 3072 columns in bf16 / fp32
+    run the tuned kernels, and only those take strided views or the gated form;
+  * gated_residual_layer_norm fuses the residual update in front of a modulated
+    LayerNorm (dit_layerspec.py:152-163) into the norm, forward and backward;
   * nothing here falls back silently: with FUSED_KERNELS on, a missing
     extension or a non-GPU tensor raises.  The eager branches below exist only
     because the reference modules select eager math when FUSED_KERNELS is off.

@@ -545,3 +545,39 @@ def test_profile_hook_brackets_the_row_kernel(capi, gpu_device):
     assert hip.hipEventElapsedTime(ctypes.byref(ms2), ev[0], ev[1]) == 0 and ms2.value == ms.value
     for e in ev:
         hip.hipEventDestroy(e)
+
+
+def test_rows_past_two_to_the_31_elements(capi, gpu_device):
+    """700 000 x 3072 = 2.15e9 elements per tensor: row offsets need 64 bits (the reference kernels index
+    with a 32-bit row*cols, adaln_backward.cu:78).  The first and the last rows are checked against eager."""
+    rows, C = 700_000, 3072
+    assert rows * C > 2 ** 31
+    gen = torch.Generator(device=gpu_device).manual_seed(5)
+    x = torch.empty(1, rows, C, device=gpu_device, dtype=torch.bfloat16)
+    grad = torch.empty_like(x)
+    for lo in range(0, rows, 100_000):     # filled in slices: no 8.6 GB fp32 temporary
+        n = min(100_000, rows - lo)
+        x[0, lo:lo + n] = torch.randn(n, C, device=gpu_device, generator=gen).bfloat16()
+        grad[0, lo:lo + n] = torch.randn(n, C, device=gpu_device, generator=gen).bfloat16()
+    scale = (0.1 * torch.randn(1, C, device=gpu_device, generator=gen)).bfloat16()
+    shift = (0.1 * torch.randn(1, C, device=gpu_device, generator=gen)).bfloat16()
+    w = (1 + 0.02 * torch.randn(C, device=gpu_device, generator=gen)).bfloat16()
+    idx = torch.cat([torch.arange(0, 8), torch.arange(rows - 8, rows)]).to(gpu_device)
+    xs, gs = x[:, idx].cpu(), grad[:, idx].cpu()
+    out, mean, rstd = capi.adaln_forward(x, scale, shift, EPS)
+    want_out, want_dx, _, _ = O.eager_adaln_fwd_bwd(xs, scale.cpu(), shift.cpu(), gs)
+    assert_fwd_bf16(out[:, idx], want_out, O.adaln_excuse(xs, scale.cpu(), shift.cpu(), want_out), "adaln out")
+    dx, ds, dh = capi.adaln_backward(grad, x, scale, mean, rstd)
+    del out
+    assert_grad_bf16(dx[:, idx], want_dx, "adaln dx", allow=1e-4)
+    want_dh = torch.zeros(C, device=gpu_device)
+    for lo in range(0, rows, 100_000):
+        want_dh += grad[0, lo:lo + 100_000].float().sum(0)
+    assert O.frac_outside(dh.cpu(), want_dh.cpu().reshape(1, C), 1e-2, 1e-2) == 0.0
+    del dx
+    out, rstd = capi.rmsnorm_forward(x[0], w, EPS)
+    want_out, want_dx, _ = O.eager_rmsnorm_fwd_bwd(xs[0], w.cpu(), gs[0])
+    assert_fwd_bf16(out[idx], want_out, None, "rms out")
+    dx, dw = capi.rmsnorm_backward(grad[0], x[0], w, rstd)
+    assert_grad_bf16(dx[idx], want_dx, "rms dx")
+    assert torch.isfinite(dw.float()).all()
