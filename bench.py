@@ -243,13 +243,24 @@ def main():
     L = capi.lib()
     calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)
     headline = args.workload == "cfg4"
+    # A step streams every tensor once.  When a tensor is smaller than twice the 256 MB last-level
+    # cache, successive steps rotate through three separately allocated buffer sets so that no step
+    # finds its inputs cached by the one before; the large workloads evict themselves.
+    buffer_sets = [calls]
+    if tensor_bytes < 512 * 2 ** 20:
+        buffer_sets += [build_workload(args.workload, torch, capi, dev)[0] for _ in range(2)]
+    turn = [0]
+
+    def next_set():
+        turn[0] += 1
+        return buffer_sets[turn[0] % len(buffer_sets)]
 
     names = [n for n, _, _ in calls]
     mults = dict((n, m) for n, _, m in calls)
 
     def step():
         """One pass of the hot path."""
-        for _, fn, _ in calls:
+        for _, fn, _ in next_set():
             fn()
 
     def per_call_profile(n_steps):
@@ -258,19 +269,24 @@ def main():
         evs = [{n: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for n in names}
                for _ in range(n_steps)]
         for k in range(n_steps):
-            for name, fn, _ in calls:
+            for name, fn, _ in next_set():
                 evs[k][name][0].record()
                 fn()
                 evs[k][name][1].record()
         torch.cuda.synchronize()
-        return {n: sum(evs[k][n][0].elapsed_time(evs[k][n][1]) for k in range(n_steps)) / n_steps for n in names}
+        return {n: sorted(evs[k][n][0].elapsed_time(evs[k][n][1]) for k in range(n_steps)) for n in names}
 
     # warm-up: W untimed steps, then (still untimed) a few more with per-call events for the breakdown
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    avg_ms = per_call_profile(10)
+    samples = per_call_profile(30)
+    avg_ms = {n: sum(v) / len(v) for n, v in samples.items()}
+    pct = lambda v, q: v[min(len(v) - 1, int(round(q * (len(v) - 1))))]
     per_call = {n: {"avg_us": round(avg_ms[n] * 1e3, 1),
+                    "p10_us": round(pct(samples[n], 0.1) * 1e3, 1),
+                    "median_us": round(pct(samples[n], 0.5) * 1e3, 1),
+                    "p90_us": round(pct(samples[n], 0.9) * 1e3, 1),
                     "GB/s": round(mults[n] * tensor_bytes / avg_ms[n] / 1e6, 1),
                     "frac_of_peak": round(mults[n] * tensor_bytes / avg_ms[n] / 1e6 / HBM_PEAK_GBS, 4)}
                 for n in names}
@@ -292,7 +308,7 @@ def main():
     arm = L.tt_norm_profile_next_row_kernel
 
     def timed_step(pair):
-        for name, fn, _ in calls:
+        for name, fn, _ in next_set():
             if name == dom:
                 arm(pair[0], pair[1])
             fn()
@@ -346,6 +362,7 @@ def main():
         "dtype": dtype_name,
         "data": "synthetic",
         "config": {"workload": WORKLOADS[args.workload], "tensor_bytes": tensor_bytes,
+                   "buffer_sets": len(buffer_sets),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "tokens_per_s": round(tokens_per_step / (ms_per_step * 1e-3), 1),
