@@ -66,13 +66,17 @@ WORKLOADS = {
 }
 
 
+# The HIP stream every call is enqueued on (looked up at call time: graph capture swaps it).
+_LAUNCH_STREAM = [None]
+
+
 def build_workload(name, torch, capi, dev):
     """Allocates the inputs of one workload in HBM and returns (calls, tensor_bytes, tokens_per_step, dtype)
     with calls = [(call name, closure, algorithmic traffic in tensors)]."""
     L = capi.lib()
     gen = torch.Generator(device=dev).manual_seed(0)
     p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
-    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    _LAUNCH_STREAM[0] = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
     def ck(st, what):
         if st != 0:
@@ -90,9 +94,9 @@ def build_workload(name, torch, capi, dev):
         out, dx, rstd, dw = torch.empty_like(x), torch.empty_like(x), f32(rows), torch.empty_like(w)
         n = L.tt_rmsnorm_backward_workspace_bytes(rows, cols, dt)
         ws = scratch(n)
-        fwd = lambda: ck(L.tt_rmsnorm_forward(p(out), p(rstd), p(x), p(w), rows, cols, EPS, dt, stream), "rms fwd")
+        fwd = lambda: ck(L.tt_rmsnorm_forward(p(out), p(rstd), p(x), p(w), rows, cols, EPS, dt, _LAUNCH_STREAM[0]), "rms fwd")
         bwd = lambda: ck(L.tt_rmsnorm_backward(p(dx), p(dw), p(grad), p(x), p(w), p(rstd), rows, cols, dt, p(ws), n,
-                                               stream), "rms bwd")
+                                               _LAUNCH_STREAM[0]), "rms bwd")
         return [("rmsnorm_forward" + tag, fwd, 2), ("rmsnorm_backward" + tag, bwd, 3)], out
 
     def adaln_pair(x, grad, scale, shift):
@@ -105,9 +109,9 @@ def build_workload(name, torch, capi, dev):
         n = L.tt_adaln_backward_workspace_bytes(batch, rps, cols, dt)
         ws = scratch(n)
         fwd = lambda: ck(L.tt_adaln_forward(p(out), p(mean), p(rstd), p(x), p(scale), p(shift), batch, rps, cols,
-                                            EPS, dt, stream), "adaln fwd")
+                                            EPS, dt, _LAUNCH_STREAM[0]), "adaln fwd")
         bwd = lambda: ck(L.tt_adaln_backward(p(dx), p(dsc), p(dsh), p(grad), p(x), p(scale), p(mean), p(rstd), batch,
-                                             rps, cols, dt, p(ws), n, stream), "adaln bwd")
+                                             rps, cols, dt, p(ws), n, _LAUNCH_STREAM[0]), "adaln bwd")
         return [("adaln_forward", fwd, 2), ("adaln_backward", bwd, 3)], out
 
     bf = torch.bfloat16
@@ -145,11 +149,11 @@ def build_workload(name, torch, capi, dev):
             ws = scratch(n)
             fwd = (lambda out=out, rstd=rstd, view=view, w=w, xs=xs:
                    ck(L.tt_rmsnorm_forward_strided(p(out), p(rstd), p(view), p(w), B, H, S, xs[0], xs[1], xs[2], D,
-                                                   EPS, capi.BF16, stream), "rms fwd strided"))
+                                                   EPS, capi.BF16, _LAUNCH_STREAM[0]), "rms fwd strided"))
             bwd = (lambda dx=dx, dw=dw, grad=grad, view=view, w=w, rstd=rstd, xs=xs, ds=ds, ws=ws, n=n:
                    ck(L.tt_rmsnorm_backward_strided(p(dx), p(dw), p(grad), p(view), p(w), p(rstd), B, H, S, xs[0],
                                                     xs[1], xs[2], ds[0], ds[1], ds[2], D, capi.BF16, p(ws), n,
-                                                    stream), "rms bwd strided"))
+                                                    _LAUNCH_STREAM[0]), "rms bwd strided"))
             calls += [("rmsnorm_forward_strided" + tag, fwd, 2), ("rmsnorm_backward_strided" + tag, bwd, 3)]
         return calls, B * H * S * D * 2, S, "bf16", mixed
     if name == "cfg5":
@@ -173,11 +177,11 @@ def build_workload(name, torch, capi, dev):
         n = L.tt_gated_residual_adaln_backward_workspace_bytes(B, S, COLS, capi.BF16)
         ws = scratch(n)
         fwd = lambda: ck(L.tt_gated_residual_adaln_forward(p(h2), p(out), p(mean), p(rstd), p(h), p(a), p(gate),
-                                                           p(scale), p(shift), B, S, COLS, EPS, capi.BF16, stream),
+                                                           p(scale), p(shift), B, S, COLS, EPS, capi.BF16, _LAUNCH_STREAM[0]),
                          "gated fwd")
         bwd = lambda: ck(L.tt_gated_residual_adaln_backward(p(dh), p(da), p(dq), p(dsc), p(dsh), p(go), p(g2), p(h2),
                                                             p(a), p(gate), p(scale), p(mean), p(rstd), B, S, COLS,
-                                                            capi.BF16, p(ws), n, stream), "gated bwd")
+                                                            capi.BF16, p(ws), n, _LAUNCH_STREAM[0]), "gated bwd")
         return [("gated_residual_adaln_forward", fwd, 4), ("gated_residual_adaln_backward", bwd, 6)], \
             S * COLS * 2, S, "bf16", h
     raise ValueError(name)
@@ -189,6 +193,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU eager timing")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="capture one step per buffer set into a HIP graph and replay it in the timed region "
+                         "(what a launch-bound caller would do; matters for the small workloads only)")
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS),
                     help="cfg4 (default) is the headline step; the others measure the remaining "
                          "configurations and the call sites around the path with the same method")
@@ -304,19 +311,36 @@ def main():
             raise RuntimeError("hipEventCreate failed")
         return e
 
-    pairs = [(hip_event(), hip_event()) for _ in range(args.steps)]
+    pairs = [] if args.hip_graph else [(hip_event(), hip_event()) for _ in range(args.steps)]
     arm = L.tt_norm_profile_next_row_kernel
+    graphs = []
+    if args.hip_graph:
+        # the entry points only launch kernels, so a step captures as is; one graph per buffer set
+        for cs in buffer_sets:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                eager_stream = _LAUNCH_STREAM[0]
+                _LAUNCH_STREAM[0] = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+                for _, fn, _ in cs:
+                    fn()
+                _LAUNCH_STREAM[0] = eager_stream
+            graphs.append(g)
+        for g in graphs:
+            g.replay()
 
-    def timed_step(pair):
+    def timed_step(k):
+        if graphs:
+            graphs[k % len(graphs)].replay()
+            return
         for name, fn, _ in next_set():
             if name == dom:
-                arm(pair[0], pair[1])
+                arm(pairs[k][0], pairs[k][1])
             fn()
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        timed_step(pairs[k])
+        timed_step(k)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
@@ -330,7 +354,8 @@ def main():
         dom_ms += ms.value
         hip.hipEventDestroy(a)
         hip.hipEventDestroy(b)
-    dom_ms /= args.steps
+    # under graph replay no event pair can be armed: the dominant call's untimed HIP-event average stands in
+    dom_ms = dom_ms / args.steps if pairs else avg_ms[dom]
     achieved = mults[dom] * tensor_bytes / (dom_ms * 1e-3) / 1e9
 
     # streaming-copy yardstick (read one tensor, write one tensor) with the same access pattern
@@ -362,7 +387,7 @@ def main():
         "dtype": dtype_name,
         "data": "synthetic",
         "config": {"workload": WORKLOADS[args.workload], "tensor_bytes": tensor_bytes,
-                   "buffer_sets": len(buffer_sets),
+                   "buffer_sets": len(buffer_sets), "hip_graph": bool(args.hip_graph),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "tokens_per_s": round(tokens_per_step / (ms_per_step * 1e-3), 1),

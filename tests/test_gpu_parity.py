@@ -418,6 +418,41 @@ def test_non_default_stream_and_output_reuse(capi, gpu_device):
     assert torch.equal(out, ref)
 
 
+def test_calls_capture_into_a_hip_graph_and_replay(capi, gpu_device):
+    """The entry points only launch kernels on the stream they are given (no allocation, no memset, no
+    synchronisation), so a caller can capture a forward+backward into a HIP graph.  Every replay, with
+    new input values and eager work in between, must equal the directly launched result bit for bit."""
+    C, S = 3072, 700
+    mk = lambda seed: O.make_adaln_inputs(2, S, C, torch.bfloat16, seed=seed)
+    static = {k: v.to(gpu_device) for k, v in mk(900).items()}
+    q = {k: v.to(gpu_device) for k, v in O.make_rmsnorm_inputs((S * 24,), 128, torch.bfloat16, seed=901).items()}
+
+    def run():
+        out, mean, rstd = capi.adaln_forward(static["x"], static["scale"], static["shift"], EPS)
+        grads = capi.adaln_backward(static["grad"], static["x"], static["scale"], mean, rstd)
+        qo, qr = capi.rmsnorm_forward(q["x"], q["weight"], EPS)
+        qg = capi.rmsnorm_backward(q["grad"], q["x"], q["weight"], qr)
+        return (out, *grads, qo, *qg)
+
+    run()                                   # warm: first-use device queries happen outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for replay in range(3):
+        fresh = mk(910 + replay)
+        for k in static:
+            static[k].copy_(fresh[k].to(gpu_device))
+        q["x"].copy_(torch.roll(q["x"], 1 + replay, 0))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = run()                        # eager launches of the same calls on the same inputs
+        torch.cuda.synchronize()
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert torch.equal(g, w), (replay, i)
+
+
 def test_error_statuses(capi, gpu_device):
     L = capi.lib()
     x = torch.zeros(8, 3072, dtype=torch.bfloat16, device=gpu_device)
