@@ -33,10 +33,10 @@ HBM_PEAK_GBS = 8000.0
 # (scaled by the same counters on the plain copy kernel); None until measured.
 MEASURED_TRAFFIC_BYTES = {
     # (FETCH_SIZE KiB * 2.000 + WRITE_SIZE KiB * 1.000) * 1024, see profiles/bench_cfg4_all_kernels.md
-    "rmsnorm_backward": int((714789.7 * 2.0 + 715874.8) * 1024),
-    "adaln_backward": int((716633.5 * 2.0 + 718944.0) * 1024),
-    "rmsnorm_forward": int((356450.6 * 2.0 + 713734.8) * 1024),
-    "adaln_forward": int((356500.1 * 2.0 + 714670.7) * 1024),
+    "rmsnorm_backward": int((714788.4 * 2.0 + 715872.0) * 1024),
+    "adaln_backward": int((716689.7 * 2.0 + 718944.0) * 1024),
+    "rmsnorm_forward": int((356452.5 * 2.0 + 713734.0) * 1024),
+    "adaln_forward": int((356500.1 * 2.0 + 714657.6) * 1024),
 }
 
 

@@ -17,10 +17,11 @@
 #include "norm_device.h"
 #include "norm_host.h"
 
-// Backward pipeline shape at 3072 columns (measured back-to-back at 118 800 rows):
-// plain loop, one row buffer; nothing but the current row in flight per wavefront.
+// Backward pipeline shape at 3072 columns (measured back-to-back at 118 800 rows, with
+// write-through stores): two row buffers, the next row requested half-way through the current
+// one: 359 us; plain loop with one row buffer 373 us; next row requested a full row ahead 384 us.
 #ifndef TTN_ADALN_BWD_ROW_BUFFERS
-#define TTN_ADALN_BWD_ROW_BUFFERS 1
+#define TTN_ADALN_BWD_ROW_BUFFERS 2
 #endif
 // Gated backward, 2-byte rows: when attn and e (the gradient arriving at h2) are fetched.
 //   0: with g and x, one row at a time
@@ -31,7 +32,16 @@
 #define TTN_GATED_OPERANDS 1
 #endif
 #ifndef TTN_ADALN_BWD_PREFETCH_MID
-#define TTN_ADALN_BWD_PREFETCH_MID 0
+#define TTN_ADALN_BWD_PREFETCH_MID 1
+#endif
+// Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
+// Backward (2 reads + 1 write): 379 -> 358 us with write-through; the gated backward (4 reads + 2 writes)
+// and the forward kernels measure the same either way and stay plain.
+#ifndef TTN_ADALN_FWD_STORE
+#define TTN_ADALN_FWD_STORE 0
+#endif
+#ifndef TTN_ADALN_BWD_STORE
+#define TTN_ADALN_BWD_STORE 1
 #endif
 // Dynamic LDS requested by the forward launch (0: none).  Only a throttle on how many
 // one-shot workgroups a compute unit holds at once; the kernel does not touch it.
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) hv[j] += av[j];
                 xr[k] = E::pack(hv);  // h2: the new residual stream, and the row that is normalised
-                if (ok) store16_stream(ph + k * LANES, xr[k]);
+                if (ok) store16<TTN_ADALN_FWD_STORE>(ph + k * LANES, xr[k]);
             }
         }
 
@@ -186,7 +196,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r as x*r + (-mu*r)
             if constexpr (WRITE_XNORM) {
                 const u32x4 xn = E::pack(v);
-                if (ok) store16_stream(pn + k * LANES, xn);
+                if (ok) store16<TTN_ADALN_FWD_STORE>(pn + k * LANES, xn);
                 E::unpack(xn, v);
             } else {
                 E::round(v);  // xn
@@ -196,7 +206,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::round(v);  // xn * (1 + scale)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] += hv[j];
-            if (ok) store16_stream(po + k * LANES, E::pack(v));
+            if (ok) store16<TTN_ADALN_FWD_STORE>(po + k * LANES, E::pack(v));
         }
     }
 }
@@ -383,7 +393,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o[j] += ev[j];
                 const u32x4 dhp = E::pack(o);  // dh: gradient of h2 = of the residual input
-                if (b.ok) store16_stream(pd + k * LANES, dhp);
+                if (b.ok) store16<0>(pd + k * LANES, dhp);
                 E::unpack(dhp, o);
                 if constexpr (kGateResident) {
 #pragma unroll
@@ -395,12 +405,12 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) av[j] *= o[j];
-                if (b.ok) store16_stream(reinterpret_cast<u32x4 *>(da + b.row * C) + l + k * LANES, E::pack(dav));
+                if (b.ok) store16<0>(reinterpret_cast<u32x4 *>(da + b.row * C) + l + k * LANES, E::pack(dav));
                 E::round(av);  // dh*attn materialised in the element type before the column sum
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
             } else {
-                if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
+                if (b.ok) store16<TTN_ADALN_BWD_STORE>(pd + k * LANES, E::pack(o));
             }
             if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
 #pragma unroll

@@ -35,6 +35,15 @@
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
+// Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
+// Backward (2 reads + 1 write): 367 -> 353 us with write-through; forward (1 read + 1 write) measures
+// the same either way and stays plain.
+#ifndef TTN_RMS_FWD_STORE
+#define TTN_RMS_FWD_STORE 0
+#endif
+#ifndef TTN_RMS_BWD_STORE
+#define TTN_RMS_BWD_STORE 1
+#endif
 
 namespace ttn {
 
@@ -146,7 +155,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::round(v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
-            if (ok) store16_stream(po + k * LANES, E::pack(v));
+            if (ok) store16<TTN_RMS_FWD_STORE>(po + k * LANES, E::pack(v));
         }
     }
 }
@@ -262,7 +271,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 o[j] = fmaf(xs, coef, gy[j] * r);
                 y[j] = FROM_OUT ? xs : xs * r;
             }
-            if (b.ok) store16_stream(pd + k * LANES, E::pack(o));
+            if (b.ok) store16<TTN_RMS_BWD_STORE>(pd + k * LANES, E::pack(o));
             E::round(y);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
