@@ -84,3 +84,26 @@ def adaln_bwd(x, scale, mean, rstd, g):
     fn(_ptr(x), _ptr(scale), _ptr(mean), _ptr(rstd), _ptr(g), _ptr(dx), _ptr(dscale), _ptr(dshift),
        acc.ctypes.data_as(ctypes.c_void_p), ctypes.c_long(B), ctypes.c_long(S), ctypes.c_long(C))
     return dx, dscale, dshift
+
+
+def gated_residual_adaln_fwd(h, attn, gate, scale, shift, eps: float):
+    """bf16 only.  Returns (h2, out, mean, rstd)."""
+    assert h.dtype == torch.bfloat16
+    B, S, C = h.shape
+    h2 = torch.empty_like(h)
+    lib().oc_gated_residual_fwd_bf16(_ptr(h), _ptr(attn), _ptr(gate), _ptr(h2), ctypes.c_long(B), ctypes.c_long(S),
+                                     ctypes.c_long(C))
+    out, mean, rstd = adaln_fwd(h2, scale, shift, eps)
+    return h2, out, mean, rstd
+
+
+def gated_residual_adaln_bwd(h2, attn, gate, scale, mean, rstd, grad_out, grad_h2=None):
+    """bf16 only.  Returns (dh, dattn, dgate, dscale, dshift)."""
+    B, S, C = h2.shape
+    dxn, dscale, dshift = adaln_bwd(h2, scale, mean, rstd, grad_out)
+    dh, dattn, dgate = torch.empty_like(h2), torch.empty_like(h2), torch.empty_like(gate)
+    acc = np.empty(C, dtype=np.float64)
+    lib().oc_gated_residual_bwd_bf16(_ptr(dxn), None if grad_h2 is None else _ptr(grad_h2), _ptr(attn), _ptr(gate),
+                                     _ptr(dh), _ptr(dattn), _ptr(dgate), acc.ctypes.data_as(ctypes.c_void_p),
+                                     ctypes.c_long(B), ctypes.c_long(S), ctypes.c_long(C))
+    return dh, dattn, dgate, dscale, dshift

@@ -253,3 +253,38 @@ void oc_adaln_bwd_f32(const float *x, const float *scale, const float *mean, con
         }
     }
 }
+
+/* ---- gated residual update in front of the AdaLN (teletron/models/dit/dit_layerspec.py:152):
+ * h2 = rnd(h + rnd(attn * gate[b])).  The norm of h2 is oc_adaln_fwd_bf16 on the result. */
+void oc_gated_residual_fwd_bf16(const uint16_t *h, const uint16_t *attn, const uint16_t *gate,
+                                uint16_t *h2, long batch, long seq, long cols) {
+    for (long b = 0; b < batch; ++b)
+        for (long s = 0; s < seq; ++s)
+            for (long c = 0; c < cols; ++c) {
+                long i = (b * seq + s) * cols + c;
+                float m = rnd_bf16(bf16_to_f32(attn[i]) * bf16_to_f32(gate[b * cols + c]));
+                h2[i] = f32_to_bf16(bf16_to_f32(h[i]) + m);
+            }
+}
+
+/* Backward of the update, given dxn = the norm's dx (bf16, from oc_adaln_bwd_bf16) and dh2 = the
+ * gradient reaching h2 from its later uses (may be NULL):
+ *   dh = rnd(dxn + dh2); dattn = rnd(dh * gate[b]); dgate[b,c] = sum_s rnd(dh * attn).
+ * acc: caller-provided double[cols] scratch. */
+void oc_gated_residual_bwd_bf16(const uint16_t *dxn, const uint16_t *dh2, const uint16_t *attn,
+                                const uint16_t *gate, uint16_t *dh, uint16_t *dattn, uint16_t *dgate,
+                                double *acc, long batch, long seq, long cols) {
+    for (long b = 0; b < batch; ++b) {
+        for (long c = 0; c < cols; ++c) acc[c] = 0.0;
+        for (long s = 0; s < seq; ++s)
+            for (long c = 0; c < cols; ++c) {
+                long i = (b * seq + s) * cols + c;
+                float d = bf16_to_f32(dxn[i]);
+                if (dh2) d = rnd_bf16(d + bf16_to_f32(dh2[i]));
+                dh[i] = f32_to_bf16(d);
+                dattn[i] = f32_to_bf16(d * bf16_to_f32(gate[b * cols + c]));
+                acc[c] += (double)rnd_bf16(d * bf16_to_f32(attn[i]));
+            }
+        for (long c = 0; c < cols; ++c) dgate[b * cols + c] = f32_to_bf16((float)acc[c]);
+    }
+}

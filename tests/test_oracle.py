@@ -341,6 +341,19 @@ def test_gated_staged_agrees_with_eager_bf16():
         assert O.frac_outside(got, want, 1e-2, 1e-3) == 0.0
     # dgate sums dh*attn, and dh is known to an ulp only: random-walk bound on the column
     assert O.colsum_outside(sdq, edq, terms * a.float(), dim=1) == 0
+    # the scalar C restatement (explicit RNE, double accumulation) tells the same story
+    ch2, cout, cmu, cr = Cc.gated_residual_adaln_fwd(h, a, q, sc, sh, EPS)
+    assert torch.equal(ch2, eh2)
+    rep = O.compare_bf16_ulp(cout, eout, excuse_abs=O.adaln_excuse(eh2, sc, sh, eout))
+    assert rep.n_gt1 == 0 and rep.n_excused < 1e-4 * rep.n and rep.frac_exact > 0.999, rep
+    for with_h2 in (True, False):
+        want = (edh, eda, edq) if with_h2 else O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, None)[2:5]
+        cdh, cda, cdq, cdsc, cdsh = Cc.gated_residual_adaln_bwd(eh2, a, q, sc, cmu, cr, go, g2 if with_h2 else None)
+        t = want[0].float().abs() + (g2.float().abs() if with_h2 else 0)
+        assert O.frac_outside(cdh, want[0], 1e-2, 1e-3, magnitude=t) < 1e-5
+        assert O.frac_outside(cda, want[1], 1e-2, 1e-3, magnitude=t * q.float().abs()[:, None]) < 1e-5
+        assert O.colsum_outside(cdq, want[2], t * a.float(), dim=1) == 0
+        assert O.frac_outside(cdsc, edsc, 1e-2, 1e-3) == 0.0 and O.frac_outside(cdsh, edsh, 1e-2, 1e-3) == 0.0
     # and the float64 truth is within bf16 rounding noise of both
     truth = O.truth_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
     assert O.frac_outside(sdh, truth[2], 2e-2, 2e-2) < 1e-4
