@@ -438,6 +438,46 @@ def Get_RMSNorm():
     return RMSNorm
 
 
+class AdaLNContinuous(nn.Module):
+    """The model's output norm (dit_layerspec.py:50-78): SiLU -> Linear -> (scale, shift), then
+    norm(x) * (1 + scale) + shift with scale, shift [B, C] broadcast as written there, i.e. along
+    x's second-to-last dimension: x is [S, B, C] (the sequence-first layout of the caller) or [B, C].
+    Same constructor arguments (config needs .hidden_size only) plus fused_kernels: with it, and
+    norm_type "layer_norm", norm and modulation run as the fused AdaLN kernel."""
+
+    def __init__(self, config, conditioning_embedding_dim: int, modulation_bias: bool = True,
+                 norm_type: str = "layer_norm", fused_kernels: bool = False):
+        super().__init__()
+        hidden = config.hidden_size
+        self.hidden_size = hidden
+        self.adaLN_modulation = nn.Sequential(nn.SiLU(), nn.Linear(conditioning_embedding_dim, hidden * 2,
+                                                                   bias=modulation_bias))
+        self.fused_kernels = bool(fused_kernels) and norm_type == "layer_norm"
+        if norm_type == "layer_norm":
+            self.norm = nn.LayerNorm(hidden, elementwise_affine=False, eps=1e-6)
+        elif norm_type == "rms_norm":
+            # the reference calls RMSNorm(hidden, eps=1e-6), which its own RMSNorm signature rejects
+            # (config is a required argument, dit_fusedlayers.py:354); built here as evidently meant
+            self.norm = RMSNorm(hidden, config, eps=1e-6)
+        else:
+            raise ValueError("Unknown normalization type {}".format(norm_type))
+        if self.fused_kernels:
+            if not cols_supported(hidden, torch.float32):
+                raise ValueError(f"fused_kernels=True: {_unsupported(hidden, torch.float32)}")
+            _require_extension(fused_adaln, "fused_adaln")
+
+    def forward(self, x: torch.Tensor, conditioning_embedding: torch.Tensor) -> torch.Tensor:
+        emb = self.adaLN_modulation(conditioning_embedding)
+        scale, shift = torch.chunk(emb, 2, dim=1)
+        if not self.fused_kernels:
+            return self.norm(x) * (1 + scale) + shift
+        if x.dim() == 3:    # [S, B, C]: the kernel wants a sample's rows together
+            return modulated_layer_norm(x.transpose(0, 1), scale, shift, eps=1e-6).transpose(0, 1)
+        if x.dim() == 2:    # [B, C]: one row per sample
+            return modulated_layer_norm(x.unsqueeze(1), scale, shift, eps=1e-6).squeeze(1)
+        raise ValueError(f"AdaLNContinuous expects x of [S, B, C] or [B, C], got {tuple(x.shape)}")
+
+
 def install_as_teletron_op() -> None:
     """Registers the extension modules under the reference's top-level names so
     that `import fused_adaln` / `import fused_rmsnorm` in unmodified reference

@@ -187,6 +187,34 @@ def test_gated_residual_function_autograd(FL, gpu_device, use_h2):
     grad_ok(leaves[4].grad, want[6])
 
 
+def test_adaln_continuous_fused_vs_eager_branch(FL, gpu_device):
+    """The output norm (dit_layerspec.py:50-78) on sequence-first input, batch 1 and batch 3."""
+    from types import SimpleNamespace
+    for B in (1, 3):
+        torch.manual_seed(5 + B)
+        S, C, E = 129, 3072, 256
+        fused = FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E, fused_kernels=True).to(gpu_device).bfloat16()
+        eager = FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E).bfloat16()
+        eager.load_state_dict({k: v.cpu() for k, v in fused.state_dict().items()})
+        x = torch.randn(S, B, C).bfloat16()
+        cond = torch.randn(B, E).bfloat16()
+        xg = x.to(gpu_device).requires_grad_(True)
+        xc = x.clone().requires_grad_(True)
+        got, want = fused(xg, cond.to(gpu_device)), eager(xc, cond)
+        assert got.shape == want.shape == (S, B, C)
+        emb = eager.adaLN_modulation(cond)
+        scale, shift = emb[:, :C].detach(), emb[:, C:].detach()
+        # the modulation rows come from a bf16 GEMM on either device: compare the norm on identical rows instead
+        ref = O.eager_adaln(x.transpose(0, 1), scale, shift, 1e-6).transpose(0, 1)
+        torch.testing.assert_close(want, ref)
+        mod = FL.modulated_layer_norm(x.to(gpu_device).transpose(0, 1), scale.to(gpu_device), shift.to(gpu_device))
+        fwd_ok(mod.transpose(0, 1), ref, O.adaln_excuse(x.transpose(0, 1), scale, shift, ref.transpose(0, 1)).transpose(0, 1))
+        assert (got.detach().cpu().float() - want.float()).abs().max() <= 0.1 * want.float().abs().max()
+        got.backward(torch.ones_like(got))
+        assert xg.grad.shape == x.shape and torch.isfinite(xg.grad.float()).all()
+        assert fused.adaLN_modulation[1].weight.grad is not None
+
+
 def test_reference_signature_extension_calls(FL, gpu_device):
     """Drive the extension exactly as the reference's autograd classes do
     (dit_fusedlayers.py:95-104,128-136,305-313,337-346)."""

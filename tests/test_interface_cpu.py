@@ -149,6 +149,27 @@ def test_adaln_zero_modules_eager_branch_matches_oracle():
         fused(x, emb=temb)
 
 
+def test_adaln_continuous_eager_branch():
+    """dit_layerspec.py:72-78: x is sequence-first [S, B, C]; scale/shift [B, C] broadcast along dim -2."""
+    from types import SimpleNamespace
+    from teletron_amd import fusedlayers as FL
+    torch.manual_seed(1)
+    S, B, C, E = 7, 3, 64, 32
+    m = FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E)
+    x, cond = torch.randn(S, B, C), torch.randn(B, E)
+    emb = m.adaLN_modulation(cond)
+    scale, shift = emb[:, :C], emb[:, C:]
+    want = O.eager_adaln(x.transpose(0, 1), scale, shift, 1e-6).transpose(0, 1)   # per-sample modulation
+    torch.testing.assert_close(m(x, cond), want)
+    r = FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E, norm_type="rms_norm")
+    assert r(x, cond).shape == x.shape
+    with pytest.raises(ValueError, match="Unknown normalization"):
+        FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E, norm_type="nope")
+    f = FL.AdaLNContinuous(SimpleNamespace(hidden_size=C), E, fused_kernels=True)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        f(x, cond)
+
+
 def test_fp32_layer_norm():
     from teletron_amd import fusedlayers as FL
     x = torch.randn(3, 64, generator=torch.Generator().manual_seed(0)).bfloat16()
