@@ -17,12 +17,14 @@
 #include "norm_host.h"
 
 // Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
-// Measured both ways per width: backward gains 1-3 % at 1536 columns and loses 2-3 % at 4096; left plain.
+// Measured both ways per width: backward gains up to 7 % with write-through for rows of up to six
+// accesses per lane (512 columns 212 -> 197 us, 1024 196 -> 186 us, 1536 184 -> 182 us) and loses 3-4 %
+// at eight and twelve (4096, 6144 columns), so the wide geometries keep the plain store.
 #ifndef TTN_ANY_FWD_STORE
 #define TTN_ANY_FWD_STORE 0
 #endif
 #ifndef TTN_ANY_BWD_STORE
-#define TTN_ANY_BWD_STORE 0
+#define TTN_ANY_BWD_STORE 1
 #endif
 
 namespace ttn {
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
                 o[j] = fmaf(xv[j], coef, gy[j] * r);
                 y[j] = xv[j] * r;
             }
-            if (ok && m.in[k]) store16<TTN_ANY_BWD_STORE>(pd + k * LANES, E::pack(o));
+            if (ok && m.in[k]) store16<(TTN_ANY_BWD_STORE && CHUNKS <= 6)>(pd + k * LANES, E::pack(o));
             E::round(y);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
                 xn[j] = fmaf(xv[j], r, nmr);
                 acc[1][k][j] += gv[j];
             }
-            if (ok && m.in[k]) store16<TTN_ANY_BWD_STORE>(pd + k * LANES, E::pack(o));
+            if (ok && m.in[k]) store16<(TTN_ANY_BWD_STORE && CHUNKS <= 6)>(pd + k * LANES, E::pack(o));
             E::round(xn);  // the normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
