@@ -161,3 +161,37 @@ def test_functions_take_other_widths_and_fp16(gpu_device):
     assert xq.grad.shape == q["x"].shape
     grad_ok(xq.grad.transpose(1, 2), want_dq, "dq")
     grad_ok(wq.grad, want_dw, "dw")
+
+
+def test_geometry_boundaries_forward_and_backward(capi, gpu_device):
+    """Row widths on both sides of every geometry switch (8, 16, 32, 64 lanes; 1, 2, 3, 4, 6, 8, 12, 16 accesses
+    per lane), with row counts that leave the last wavefront partly empty."""
+    pieces = [1, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 383, 384, 385,
+              511, 512, 513, 767, 768, 769, 1023, 1024]
+    for i, p in enumerate(pieces):
+        cols = p * 8
+        rows = 3 + (i * 7) % 11
+        d = O.make_rmsnorm_inputs((rows,), cols, BF, seed=800 + i)
+        want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+        x, w, g = (d[k].to(gpu_device) for k in ("x", "weight", "grad"))
+        out, rstd = capi.rmsnorm_forward(x, w, EPS)
+        fwd_16bit_ok(out, want_out, O.rmsnorm_excuse(want_out), f"rms out cols={cols}")
+        dx, dw = capi.rmsnorm_backward(g, x, w, rstd)
+        grad_ok(dx, want_dx, f"rms dx cols={cols}")
+        colsum_ok(dw, want_dw, d["grad"].float() * want_out.float(), 0, f"rms dw cols={cols}")
+        a = O.make_adaln_inputs(2, rows, cols, BF, seed=900 + i)
+        a_out, a_dx, a_ds, a_dh = O.eager_adaln_fwd_bwd(a["x"], a["scale"], a["shift"], a["grad"])
+        ax, asc, ash, ag = (a[k].to(gpu_device) for k in ("x", "scale", "shift", "grad"))
+        out, mean, rstd = capi.adaln_forward(ax, asc, ash, EPS)
+        if cols >= 64:   # a row of 8 or 56 elements has no meaningful 1-ulp statistics (xn is O(1) with 3 bits of x)
+            fwd_16bit_ok(out, a_out, O.adaln_excuse(a["x"], a["scale"], a["shift"], a_out), f"adaln out cols={cols}")
+        dx, ds, dh = capi.adaln_backward(ag, ax, asc, mean, rstd)
+        terms = O.adaln_dx_terms(a["x"], a["scale"], a["grad"])
+        # eager on the CPU keeps mean and rstd of a 16-bit row in 16 bits: a stray element of these tiny
+        # tensors may sit just outside the bar; none may be far outside
+        assert O.frac_outside(dx.cpu(), a_dx, 1e-2, 1e-3, magnitude=terms) * a_dx.numel() <= max(2, 2e-4 * a_dx.numel()), \
+            f"adaln dx cols={cols}"
+        assert O.frac_outside(dx.cpu(), a_dx, 3e-2, 3e-3, magnitude=terms) == 0.0, f"adaln dx cols={cols}"
+        colsum_ok(dh, a_dh, a["grad"].float(), 1, f"adaln dshift cols={cols}")
+        xn = torch.nn.functional.layer_norm(a["x"].float(), (cols,), None, None, EPS)
+        colsum_ok(ds, a_ds, a["grad"].float() * xn, 1, f"adaln dscale cols={cols}")
