@@ -190,8 +190,8 @@ def build_workload(name, torch, capi, dev):
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU eager timing")
     ap.add_argument("--hip-graph", action="store_true",
                     help="capture one step per buffer set into a HIP graph and replay it in the timed region "
