@@ -202,9 +202,10 @@ def parse_args():
     return ap.parse_args()
 
 
-def cpu_eager_baseline(sample_rows: int = 8192, reps: int = 3):
-    """The reference's eager formulas (oracle restatement) on the host cores, on a row
-    sample of the same workload; returns GB/s in the same algorithmic-bytes accounting."""
+def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
+    """The reference's eager formulas (oracle restatement) on the host cores, over the rows of the
+    same workload (all of them by default: about ten seconds of CPU work); returns GB/s in the same
+    algorithmic-bytes accounting."""
     import torch
     from oracle import norm_oracle as O
 
