@@ -46,9 +46,11 @@
 // Dynamic LDS requested by the forward launch (0: none).  Only a throttle on how many
 // one-shot workgroups a compute unit holds at once; the kernel does not touch it.
 // AdaLN forward spends longer in the ALU per row than RMSNorm forward and wants all the
-// wavefronts its registers allow (16 per compute unit), so no throttle here.
+// wavefronts its registers allow (16 per compute unit), so no throttle for 2-byte rows.  4-byte
+// rows carry twice the bytes per wavefront: 40 KiB on top of the 24 KiB of staged modulation rows
+// leaves two workgroups per compute unit (232 vs 244 us at 59 400 rows).
 #ifndef TTN_ADALN_FWD_DYN_LDS
-#define TTN_ADALN_FWD_DYN_LDS 0
+#define TTN_ADALN_FWD_DYN_LDS (C >= 1024 && sizeof(T) == 4 ? 40960 : 0)
 #endif
 // Backward row fetch: all of g's accesses, then all of x's (two contiguous 6 KiB runs per
 // wavefront at 3072 columns) rather than alternating 1 KiB pieces; worth ~0.7 %.

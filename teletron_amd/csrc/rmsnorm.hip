@@ -24,8 +24,10 @@
 // compute unit hold three one-shot workgroups (12 wavefronts, ~72 KiB of reads in flight),
 // which streams 5 % faster than the five its registers would allow (232 vs 244 us at
 // 118 800 rows).  The kernel does not touch this memory; it is only an occupancy throttle.
+// 4-byte rows carry twice the bytes per wavefront: two workgroups per compute unit (75 KiB each;
+// 234 vs 253 us at 59 400 rows).
 #ifndef TTN_RMS_FWD_DYN_LDS
-#define TTN_RMS_FWD_DYN_LDS (C >= 1024 && sizeof(T) == 2 ? 51200 : 0)
+#define TTN_RMS_FWD_DYN_LDS (C >= 1024 ? (sizeof(T) == 2 ? 51200 : 76800) : 0)
 #endif
 // Backward row fetch: all of g's accesses, then all of x's (two contiguous 6 KiB runs per
 // wavefront at 3072 columns) rather than alternating 1 KiB pieces; worth ~0.7 %.
