@@ -432,6 +432,89 @@ class RMSNorm(nn.Module):
         return self._norm(x.float()).type_as(x) * self.weight
 
 
+class QKVSplitNormFunction(Function):
+    """(q, k, v) = apply(mixed_qkv, weight_q, weight_k, epsilon)
+
+    mixed_qkv is the fused QKV projection as the attention module views it, [B, S, H, 3*D] with q, k, v
+    of one head side by side (dit_attention.py:149-190 with one query head per group).  q and k come
+    back RMS-normalised over D as contiguous [B, H, S, D] tensors, v as the transposed view of its
+    slice -- what torch.split, .transpose(1, 2), q_layernorm and k_layernorm produce together
+    (dit_attention.py:191-214) -- read straight out of mixed_qkv.
+    Backward writes the gradients of q and k from the kernels directly into their slices of one
+    [B, S, H, 3*D] gradient tensor and copies the gradient of v into its slice, so the concatenation
+    that torch.split's backward would run over three separate gradients never happens.
+    D must be 128 or 3072, dtype bfloat16 or float32."""
+
+    @staticmethod
+    def forward(ctx, mixed_qkv, weight_q, weight_k, epsilon):
+        ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
+        _require_gpu(mixed_qkv, "QKVSplitNormFunction")
+        if mixed_qkv.dim() != 4 or mixed_qkv.shape[-1] % 3:
+            raise ValueError(f"mixed_qkv must be [B, S, H, 3*D], got {tuple(mixed_qkv.shape)}")
+        cols = mixed_qkv.shape[-1] // 3
+        if cols not in TUNED_COLS or mixed_qkv.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"QKVSplitNormFunction needs D in {TUNED_COLS} and bfloat16/float32, got D={cols}, "
+                             f"{mixed_qkv.dtype}")
+        if weight_q.numel() != cols or weight_k.numel() != cols:
+            raise ValueError(f"weights must have {cols} elements")
+        mixed = mixed_qkv if mixed_qkv.is_contiguous() and mixed_qkv.data_ptr() % 16 == 0 else \
+            _aligned_contiguous(mixed_qkv)
+        q_in, k_in, v_in = (mixed[..., i * cols:(i + 1) * cols].transpose(1, 2) for i in range(3))
+        ws = [w.contiguous().to(mixed.dtype) for w in (weight_q, weight_k)]
+        B, H, S, _ = q_in.shape
+        outs, stats = [], []
+        for x, w in ((q_in, ws[0]), (k_in, ws[1])):
+            out = torch.empty((B, H, S, cols), dtype=mixed.dtype, device=mixed.device)
+            invvar = torch.empty(B * H * S, device=mixed.device, dtype=torch.float32)
+            ext.torch_launch_rms_forward_strided(out, x, w, float(epsilon), invvar)
+            outs.append(out)
+            stats.append(invvar)
+        ctx.save_for_backward(mixed, ws[0], ws[1], stats[0], stats[1])
+        ctx.cols = cols
+        ctx.w_meta = [(w.shape, w.dtype) for w in (weight_q, weight_k)]
+        ctx.set_materialize_grads(False)
+        # v leaves as a copy-free view only when mixed_qkv itself was usable in place
+        v_out = v_in if mixed is mixed_qkv else v_in.clone()
+        return outs[0], outs[1], v_out
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k, grad_v):
+        mixed, wq, wk, rstd_q, rstd_k = ctx.saved_tensors
+        cols = ctx.cols
+        d_mixed = torch.empty_like(mixed)
+        slices = [d_mixed[..., i * cols:(i + 1) * cols].transpose(1, 2) for i in range(3)]
+        grads_w = []
+        for i, (g, w, rstd) in enumerate(((grad_q, wq, rstd_q), (grad_k, wk, rstd_k))):
+            dw = torch.empty_like(w)
+            if g is None:
+                slices[i].zero_()
+                dw.zero_()
+            else:
+                g = _aligned_contiguous(g.to(mixed.dtype))
+                x = mixed[..., i * cols:(i + 1) * cols].transpose(1, 2)
+                fused_rmsnorm.torch_launch_rms_backward_strided(slices[i], dw, g, x, w, rstd)
+            shape, dtype = ctx.w_meta[i]
+            grads_w.append(dw.reshape(shape).to(dtype))
+        if grad_v is None:
+            slices[2].zero_()
+        else:
+            slices[2].copy_(grad_v)
+        return d_mixed, grads_w[0], grads_w[1], None
+
+
+def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSNorm"):
+    """query, key, value as `[B, H, S, D]` from the fused projection `[B, S, H, 3*D]`: the split, the
+    transposes and the two per-head RMSNorms of dit_attention.py:149-214 in one call.  Fused when
+    FUSED_KERNELS is on and the head dimension is one the tuned kernels take; the reference's own
+    sequence of operations otherwise."""
+    D = mixed_qkv.shape[-1] // 3
+    if (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in (torch.bfloat16, torch.float32)
+            and q_norm.eps == k_norm.eps):
+        return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
+    query, key, value = torch.split(mixed_qkv, [D, D, D], dim=3)
+    return q_norm(query.transpose(1, 2)), k_norm(key.transpose(1, 2)), value.transpose(1, 2)
+
+
 def Get_RMSNorm():
     """Returns the RMSNorm class (the reference hands the class out through a
     factory, dit_fusedlayers.py:350-375)."""

@@ -296,6 +296,62 @@ def test_rmsnorm_function_reads_qkv_view_in_place(FL, gpu_device):
     assert O.frac_outside(got[3].cpu(), want[3], 2e-2, 1e-3) == 0.0
 
 
+@pytest.mark.parametrize("B,S,H", [(1, 1001, 24), (2, 37, 6)])
+def test_qkv_split_norm_function_matches_the_callers_sequence(FL, gpu_device, B, S, H):
+    """torch.split + transpose + q_layernorm / k_layernorm (dit_attention.py:149-214) as one Function; the
+    gradient of the fused projection is assembled in place."""
+    D = 128
+    gen = torch.Generator().manual_seed(77 + S)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()
+    wq = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    wk = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    gq, gk, gv = (torch.randn(B, H, S, D, generator=gen).bfloat16() for _ in range(3))
+    # the caller's sequence on the CPU
+    m_c = mixed.clone().requires_grad_(True)
+    wq_c, wk_c = wq.clone().requires_grad_(True), wk.clone().requires_grad_(True)
+    q_c, k_c, v_c = torch.split(m_c, [D, D, D], dim=3)
+    q_c, k_c, v_c = O.eager_rmsnorm(q_c.transpose(1, 2), wq_c), O.eager_rmsnorm(k_c.transpose(1, 2), wk_c), v_c.transpose(1, 2)
+    torch.autograd.backward([q_c, k_c, v_c], [gq, gk, gv])
+    # fused
+    m_g = mixed.to(gpu_device).requires_grad_(True)
+    wq_g, wk_g = wq.to(gpu_device).requires_grad_(True), wk.to(gpu_device).requires_grad_(True)
+    q_g, k_g, v_g = FL.QKVSplitNormFunction.apply(m_g, wq_g, wk_g, EPS)
+    assert q_g.is_contiguous() and k_g.is_contiguous() and q_g.shape == (B, H, S, D)
+    fwd_ok(q_g, q_c.detach(), O.rmsnorm_excuse(q_c.detach()))
+    fwd_ok(k_g, k_c.detach(), O.rmsnorm_excuse(k_c.detach()))
+    assert torch.equal(v_g.detach().cpu(), v_c.detach())
+    torch.autograd.backward([q_g, k_g, v_g], [gq.to(gpu_device), gk.to(gpu_device), gv.to(gpu_device)])
+    assert m_g.grad.shape == mixed.shape and m_g.grad.is_contiguous()
+    grad_ok(m_g.grad, m_c.grad)
+    grad_ok(wq_g.grad, wq_c.grad)
+    grad_ok(wk_g.grad, wk_c.grad)
+    # v unused downstream: its slice of the gradient is zero, q and k unchanged
+    m2 = mixed.to(gpu_device).requires_grad_(True)
+    q2, k2, _ = FL.QKVSplitNormFunction.apply(m2, wq_g.detach(), wk_g.detach(), EPS)
+    torch.autograd.backward([q2, k2], [gq.to(gpu_device), gk.to(gpu_device)])
+    assert not m2.grad[..., 2 * D:].any()
+    assert torch.equal(m2.grad[..., :2 * D], m_g.grad[..., :2 * D])
+    # the module-level helper takes the same path when the switch is on
+    import os
+    qn, kn = FL.RMSNorm(D).to(gpu_device).bfloat16(), FL.RMSNorm(D).to(gpu_device).bfloat16()
+    with torch.no_grad():
+        qn.weight.copy_(wq)
+        kn.weight.copy_(wk)
+    old = os.environ.get("FUSED_KERNELS")
+    try:
+        os.environ["FUSED_KERNELS"] = "1"
+        q3, k3, v3 = FL.split_qkv_and_norm(mixed.to(gpu_device), qn, kn)
+        os.environ["FUSED_KERNELS"] = "0"
+        q4, k4, v4 = FL.split_qkv_and_norm(mixed.to(gpu_device), qn, kn)
+    finally:
+        if old is None:
+            os.environ.pop("FUSED_KERNELS", None)
+        else:
+            os.environ["FUSED_KERNELS"] = old
+    assert torch.equal(q3, q_g.detach()) and torch.equal(k3, k_g.detach()) and torch.equal(v3, v4)
+    fwd_ok(q4, q_c.detach(), O.rmsnorm_excuse(q_c.detach()))
+
+
 def test_empty_and_unaligned_inputs(FL, gpu_device):
     """Zero rows: forward returns an empty tensor, backward returns zero parameter gradients.
     A contiguous slice that starts at an odd element is copied to an aligned buffer, not rejected."""
