@@ -169,6 +169,15 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                  int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* tt_adaln_backward for an input that has another consumer (the residual stream continues past the
+ * norm, teletron/models/dit/dit_layerspec.py:126-131,152): dres [rows, cols] is the gradient the input
+ * receives from that consumer, and dx = round(round(dx of the norm) + dres), the sum autograd would
+ * otherwise form in a separate pass.  Same scratch as tt_adaln_backward.  cols must be 3072. */
+int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *dout, const void *dres,
+                               const void *x, const void *scale, const float *mean, const float *rstd,
+                               int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 /* ----------------------------------------------- gated residual + AdaLN
  * The transformer blocks update the residual stream and then normalise it:
  *     h2  = round(h + round(attn * gate[b]))

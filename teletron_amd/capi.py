@@ -25,7 +25,7 @@ EXPORTS = (
     "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
     "tt_norm_profile_next_row_kernel",
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
-    "tt_gated_residual_adaln_backward",
+    "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual",
 )
 
 
@@ -68,6 +68,7 @@ def lib() -> ctypes.CDLL:
         L.tt_gated_residual_adaln_backward_workspace_bytes.restype = sz
         L.tt_gated_residual_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
         L.tt_gated_residual_adaln_backward.argtypes = [vp] * 13 + [i64, i64, i64, ci, vp, sz, vp]
+        L.tt_adaln_backward_residual.argtypes = [vp] * 9 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
         L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
@@ -228,6 +229,25 @@ def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False):
             _check(L.tt_adaln_backward(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(x), _p(scale), _p(mean),
                                        _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n, _stream(x)),
                    "tt_adaln_backward")
+    return dx, dscale, dshift
+
+
+def adaln_backward_residual(dout, dres, x, scale, mean, rstd):
+    """AdaLN backward with the input's other gradient added in: returns (dx + dres, dscale, dshift)."""
+    _dense_gpu(dout, dres, x, scale, mean, rstd)
+    cols = x.shape[-1]
+    batch = scale.numel() // cols
+    rows = x.numel() // cols
+    dx = torch.empty_like(x)
+    dscale = torch.empty_like(scale)
+    dshift = torch.empty_like(scale)
+    with torch.cuda.device(x.device):
+        L = lib()
+        n = L.tt_adaln_backward_workspace_bytes(batch, rows // batch, cols, _dt(x))
+        ws = _workspace(n, x)
+        _check(L.tt_adaln_backward_residual(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(dres), _p(x), _p(scale),
+                                            _p(mean), _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n,
+                                            _stream(x)), "tt_adaln_backward_residual")
     return dx, dscale, dshift
 
 

@@ -226,7 +226,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // dh = rnd(rnd(dx of the norm) + e) with e the gradient arriving at h2 from its other use (may be
 // absent), written to dx; additionally da = rnd(dh * gate[b]) is written and
 // dgate[b] += rnd(dh * attn) is accumulated as a third set of column sums.
-template <typename T, int C, bool FROM_XNORM, bool GATED>
+//
+// RES = true (plain AdaLN whose input has another consumer): e is the gradient the input receives from
+// that consumer, and dx = rnd(rnd(dx of the norm) + e) -- the sum autograd would form in a pass of its own.
+template <typename T, int C, bool FROM_XNORM, bool GATED, bool RES = false>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void adaln_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
@@ -234,6 +237,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const T *__restrict__ attn, const T *__restrict__ gate, int64_t rows_per_sample,
     int blocks_per_sample) {
     static_assert(!(GATED && FROM_XNORM), "the gated form works from the saved h2");
+    static_assert(!(GATED && RES), "the gated form handles e itself");
     constexpr int NSETS = GATED ? 3 : 2;
     using G = RowGeom<T, C>;
     using E = Elem<T>;
@@ -278,7 +282,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 
     struct RowRegs {
         u32x4 g[CHUNKS], x[CHUNKS];
-        u32x4 a[kEarlyOperands ? CHUNKS : 1], e[kEarlyOperands ? CHUNKS : 1];
+        u32x4 a[kEarlyOperands ? CHUNKS : 1], e[(kEarlyOperands || RES) ? CHUNKS : 1];
         float r, mu;
         int64_t row;
         bool ok;
@@ -301,6 +305,11 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         }
 #endif
+        if constexpr (RES) {
+            const u32x4 *pe = reinterpret_cast<const u32x4 *>(e + b.row * C) + l;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.e[k] = b.ok ? load16_stream(pe + k * LANES) : u32x4{0, 0, 0, 0};
+        }
         if constexpr (kEarlyOperands) {  // otherwise these two are fetched where they are used
             const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + b.row * C) + l;
             const u32x4 *pe = reinterpret_cast<const u32x4 *>(e + b.row * C) + l;
@@ -412,6 +421,13 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
             } else {
+                if constexpr (RES) {
+                    float ev[VEC];
+                    E::round(o);  // the norm's dx, materialised in the element type
+                    E::unpack(b.e[k], ev);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) o[j] += ev[j];
+                }
                 if (b.ok) store16<TTN_ADALN_BWD_STORE>(pd + k * LANES, E::pack(o));
             }
             if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
@@ -487,7 +503,7 @@ static RowPlan adaln_backward_plan(int64_t batch, int64_t rows_per_sample, int c
     return make_row_plan(batch, rows_per_sample, RowGeom<T, C>::RPW, AdalnTune<T, C>::kBwdBlocksPerCu, cus);
 }
 
-template <typename T, int C, bool FROM_XNORM, bool GATED = false>
+template <typename T, int C, bool FROM_XNORM, bool GATED = false, bool RES = false>
 static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g, const void *xin,
                             const void *scale, const float *mean, const float *rstd, int dtype,
                             void *ws, size_t ws_bytes, const AdalnArgs &a, void *dgate = nullptr,
@@ -506,7 +522,7 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
     {
         RowKernelProfile prof(a.stream);
-        adaln_bwd_kernel<T, C, FROM_XNORM, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
+        adaln_bwd_kernel<T, C, FROM_XNORM, GATED, RES><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
             (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
             (T *)gp.h2_or_da, (const T *)gp.e, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample,
             p.blocks_per_sample);
@@ -676,6 +692,27 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                                            workspace, workspace_bytes, a, dgate, gp);
     return adaln_backward_t<float, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
                                                       workspace, workspace_bytes, a, dgate, gp);
+}
+
+/* ---- AdaLN backward with the input's other gradient added in (3072 columns) ---- */
+
+int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *dout, const void *dres,
+                               const void *x, const void *scale, const float *mean, const float *rstd,
+                               int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                               void *workspace, size_t workspace_bytes, void *stream) {
+    int st = check_adaln_args("tt_adaln_backward_residual", batch, rows_per_sample, cols, dtype,
+                              {dx, dout, dres, x, scale}, true);
+    if (st != TT_NORM_OK) return st;
+    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_adaln_backward_residual: built for cols 3072 only");
+    if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
+        return fail(TT_NORM_EINVAL, "tt_adaln_backward_residual: null dscale/dshift/mean/rstd");
+    const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
+    const GatedPtrs gp{nullptr, dres, nullptr, nullptr};
+    if (dtype == TT_NORM_BF16)
+        return adaln_backward_t<bf16_t, 3072, false, false, true>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype,
+                                                                  workspace, workspace_bytes, a, nullptr, gp);
+    return adaln_backward_t<float, 3072, false, false, true>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype,
+                                                             workspace, workspace_bytes, a, nullptr, gp);
 }
 
 }  // extern "C"

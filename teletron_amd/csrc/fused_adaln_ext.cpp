@@ -119,6 +119,35 @@ void torch_launch_adaln_backward_x(torch::Tensor &dinp, torch::Tensor &dscale, t
     adaln_backward_impl(dinp, dscale, dshift, dout, input, scale, &mean, inv_variance, rows, cols);
 }
 
+// Native backward for an input with another consumer: `dres` is the gradient the input receives from it,
+// dinp = dx of the norm + dres.  No counterpart in the reference's module.
+void torch_launch_adaln_backward_residual(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
+                                          const torch::Tensor &dout, const torch::Tensor &dres,
+                                          const torch::Tensor &input, const torch::Tensor &scale,
+                                          const torch::Tensor &mean, const torch::Tensor &inv_variance,
+                                          int64_t rows, int64_t cols) {
+    const auto dev = dout.device();
+    for (auto *t : {&dinp, &dscale, &dshift}) check_dense_on(*t, dev, "output tensor");
+    for (auto *t : {&dout, &dres, &input, &scale, &mean, &inv_variance}) check_dense_on(*t, dev, "input tensor");
+    const AdalnShape s = adaln_shape(dout, scale, rows, cols);
+    const auto st = dout.scalar_type();
+    for (auto *t : {&dout, &dres, &input}) check_elems(*t, rows * cols, st, "dout/dres/input");
+    check_elems(dinp, rows * cols, st, "dinp");
+    check_elems(scale, scale.numel(), st, "scale");
+    for (auto *t : {&dscale, &dshift}) check_elems(*t, scale.numel(), st, "dscale/dshift");
+    check_elems(mean, rows, at::kFloat, "mean");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_adaln_backward_workspace_bytes(s.batch, s.rows_per_sample, cols, s.dt);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported AdaLN shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    raise_on(tt_adaln_backward_residual(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(),
+                                        dres.data_ptr(), input.data_ptr(), scale.data_ptr(),
+                                        mean.data_ptr<float>(), inv_variance.data_ptr<float>(), s.batch,
+                                        s.rows_per_sample, cols, s.dt, ws.data_ptr(), need, current_stream(dout)),
+             "tt_adaln_backward_residual");
+}
+
 // Gated residual update fused with the norm that follows it:
 // h2 = input + attn * gate[b];  output = AdaLN(h2).  No counterpart in the reference's module.
 void torch_launch_gated_adaln_forward(torch::Tensor &h2, torch::Tensor &output, const torch::Tensor &input,
@@ -183,6 +212,8 @@ void torch_launch_gated_adaln_backward(torch::Tensor &dinp, torch::Tensor &dattn
 }
 
 PYBIND11_MODULE(fused_adaln, m) {
+    m.def("torch_launch_adaln_backward_residual", &torch_launch_adaln_backward_residual,
+          "AdaLN backward kernel with the input's other gradient added in");
     m.def("torch_launch_gated_adaln_forward", &torch_launch_gated_adaln_forward,
           "gated residual update + AdaLN forward kernel");
     m.def("torch_launch_gated_adaln_backward", &torch_launch_gated_adaln_backward,

@@ -157,6 +157,63 @@ class AdaLNModelFunction(Function):
         return grad_input, grad_scale, grad_shift, None, None
 
 
+class AdaLNResidualFunction(Function):
+    """(x_same, out) = apply(x, scale, shift, epsilon): out is AdaLNModelFunction's result and x_same is x
+    itself, handed back as an output for the caller to continue the residual stream with
+    (dit_layerspec.py:126-131 then :152).  Routing the stream through the Function lets backward add the
+    gradient it collected downstream to the norm's dx inside the kernel, in place of the separate
+    accumulation pass autograd runs when a tensor has two consumers.  3072 columns, bfloat16 / float32."""
+
+    @staticmethod
+    def forward(ctx, x, scale, shift, epsilon):
+        ext = _require_extension(fused_adaln, "fused_adaln")
+        _require_gpu(x, "AdaLNResidualFunction")
+        cols = x.shape[-1]
+        if cols != 3072 or x.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"AdaLNResidualFunction needs 3072 columns in bfloat16/float32, got {cols}, {x.dtype}")
+        x_c = _aligned_contiguous(x)
+        scale_c, shift_c = scale.contiguous().to(x.dtype), shift.contiguous().to(x.dtype)
+        if scale_c.numel() % cols or shift_c.numel() != scale_c.numel():
+            raise ValueError("scale and shift must each hold [B, cols] elements")
+        batch = scale_c.numel() // cols
+        if batch > 1 and (x.dim() < 2 or x.shape[0] != batch):
+            raise ValueError(f"{batch} modulation rows need x.shape[0] == {batch}, got {tuple(x.shape)}")
+        rows = x_c.numel() // cols
+        out = torch.empty_like(x_c)
+        mean = torch.empty(rows, device=x.device, dtype=torch.float32)
+        invvar = torch.empty(rows, device=x.device, dtype=torch.float32)
+        ext.torch_launch_adaln_forward_stats(out, x_c, scale_c, shift_c, rows, cols, float(epsilon), mean, invvar)
+        ctx.save_for_backward(x_c, scale_c, mean, invvar)
+        ctx.rows, ctx.cols = rows, cols
+        ctx.mod_shape, ctx.mod_dtype = scale.shape, scale.dtype
+        ctx.set_materialize_grads(False)
+        return x, out
+
+    @staticmethod
+    def backward(ctx, grad_x_same, grad_out):
+        x, scale_c, mean, invvar = ctx.saved_tensors
+        if grad_out is None:   # only the stream was used: the Function was an identity
+            return grad_x_same, None, None, None
+        grad_out = _aligned_contiguous(grad_out.to(x.dtype))
+        grad_input = torch.empty_like(x)
+        grad_scale, grad_shift = torch.empty_like(scale_c), torch.empty_like(scale_c)
+        if grad_x_same is None:
+            fused_adaln.torch_launch_adaln_backward_x(grad_input, grad_scale, grad_shift, grad_out, x, scale_c, mean,
+                                                      invvar, ctx.rows, ctx.cols)
+        else:
+            fused_adaln.torch_launch_adaln_backward_residual(grad_input, grad_scale, grad_shift, grad_out,
+                                                             _aligned_contiguous(grad_x_same.to(x.dtype)), x, scale_c,
+                                                             mean, invvar, ctx.rows, ctx.cols)
+        return (grad_input, grad_scale.reshape(ctx.mod_shape).to(ctx.mod_dtype),
+                grad_shift.reshape(ctx.mod_shape).to(ctx.mod_dtype), None)
+
+
+def modulated_layer_norm_keeping_stream(x, scale, shift, eps: float = 1e-6):
+    """Returns (x, LayerNorm(x) * (1 + scale[:, None]) + shift[:, None]); use the returned x for the residual
+    connection so that its gradient is added inside the norm's backward kernel."""
+    return AdaLNResidualFunction.apply(x, scale, shift, eps)
+
+
 class AdaLNCustom(nn.Module):
     """Module form of AdaLNModelFunction (dit_fusedlayers.py:139-153)."""
 

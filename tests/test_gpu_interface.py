@@ -163,6 +163,45 @@ def test_modulated_layer_norm_matches_unfused_norm2_site(FL, gpu_device):
     fwd_ok(got, want, O.adaln_excuse(d["x"], d["scale"], d["shift"], want))
 
 
+def test_adaln_keeping_the_residual_stream(FL, gpu_device):
+    """norm1 + modulate with hidden_states continuing as the residual (dit_layerspec.py:126-131, :152): the
+    stream's downstream gradient is added inside the backward kernel."""
+    d = O.make_adaln_inputs(2, 301, 3072, torch.bfloat16, seed=61)
+    g_res = O.make_adaln_inputs(2, 301, 3072, torch.bfloat16, seed=62)["grad"] * 0.5
+    xc = d["x"].clone().requires_grad_(True)
+    sc, sh = d["scale"].clone().requires_grad_(True), d["shift"].clone().requires_grad_(True)
+    out_c = O.eager_adaln(xc, sc, sh)
+    torch.autograd.backward([out_c, xc * 1.0], [d["grad"], g_res])       # x has two consumers
+    x = d["x"].to(gpu_device).requires_grad_(True)
+    s1, s2 = d["scale"].to(gpu_device).requires_grad_(True), d["shift"].to(gpu_device).requires_grad_(True)
+    x_same, out = FL.modulated_layer_norm_keeping_stream(x, s1, s2, EPS)
+    assert x_same.data_ptr() == x.data_ptr() and torch.equal(x_same, x)
+    fwd_ok(out, out_c.detach(), O.adaln_excuse(d["x"], d["scale"], d["shift"], out_c.detach()))
+    torch.autograd.backward([out, x_same * 1.0], [d["grad"].to(gpu_device), g_res.to(gpu_device)])
+    # the sum is rounded again: where the two implementations' dx differ by one ulp (0.8 % at most), the
+    # rounded sums can differ by two, so: the plain bar on all but 2e-3 of elements, twice the bar everywhere;
+    # the exact statement is the bit-identity with "plain backward, then add" below
+    terms = O.adaln_dx_terms(d["x"], d["scale"], d["grad"]) + g_res.float().abs()
+    assert O.frac_outside(x.grad.cpu(), xc.grad, 1e-2, 1e-3, magnitude=terms) <= 2e-3
+    assert O.frac_outside(x.grad.cpu(), xc.grad, 2e-2, 2e-3, magnitude=terms) == 0.0
+    grad_ok(s1.grad, sc.grad)
+    grad_ok(s2.grad, sh.grad)
+    # bit-identical to the plain backward followed by the addition
+    from teletron_amd import capi
+    _, mean, rstd = capi.adaln_forward(x.detach(), s1.detach(), s2.detach(), EPS)
+    dx_plain, _, _ = capi.adaln_backward(d["grad"].to(gpu_device), x.detach(), s1.detach(), mean, rstd)
+    assert torch.equal(x.grad, dx_plain + g_res.to(gpu_device))
+    # stream unused downstream / norm unused downstream
+    x2 = d["x"].to(gpu_device).requires_grad_(True)
+    _, out2 = FL.modulated_layer_norm_keeping_stream(x2, s1.detach(), s2.detach(), EPS)
+    out2.backward(d["grad"].to(gpu_device))
+    assert torch.equal(x2.grad, dx_plain)
+    x3 = d["x"].to(gpu_device).requires_grad_(True)
+    same3, _ = FL.modulated_layer_norm_keeping_stream(x3, s1.detach(), s2.detach(), EPS)
+    same3.backward(g_res.to(gpu_device))
+    assert torch.equal(x3.grad, g_res.to(gpu_device))
+
+
 @pytest.mark.parametrize("use_h2", [True, False])
 def test_gated_residual_function_autograd(FL, gpu_device, use_h2):
     """hidden = hidden + attn * gate.unsqueeze(1); norm2(hidden) * (1 + scale[:, None]) + shift[:, None]

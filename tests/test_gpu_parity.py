@@ -254,6 +254,11 @@ def test_full_size_adaln_properties(capi, gpu_device):
     # dshift = column sums of the upstream gradient
     want_dh = grad.float().sum(1)
     assert O.frac_outside(dh.cpu(), want_dh.cpu(), 1e-2, 1e-3) == 0.0
+    # the input's other gradient added inside the kernel == plain backward, then the addition
+    other = (0.5 * torch.randn(1, rows, C, device=gpu_device, generator=gen)).bfloat16()
+    dxr, dsr, dhr = capi.adaln_backward_residual(grad, other, x, scale, mean, rstd)
+    assert torch.equal(dxr, dx + other) and torch.equal(dsr, ds) and torch.equal(dhr, dh)
+    del dxr, other
     idx = torch.arange(0, rows, 991, device=gpu_device)
     d = {"x": x[:, idx].cpu(), "scale": scale.cpu(), "shift": shift.cpu(), "grad": grad[:, idx].cpu()}
     want_out, want_dx, _, _ = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
