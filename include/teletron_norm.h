@@ -1,6 +1,6 @@
 /* teletron_norm.h -- C ABI of the gfx950 fused normalization library
  * (libteletron_norm.so): fused RMSNorm and fused AdaLayerNorm, forward and
- * backward.  Tuned kernels for bf16 and fp32 rows of 128 or 3072 columns (the
+ * backward.  Tuned kernels for bf16, fp16 and fp32 rows of 128 or 3072 columns (the
  * shapes the reference's kernels are built for, teletron/models/dit/
  * dit_fusedlayers.py:91,301); any-width kernels for every other row of whole
  * 16-byte pieces, bf16 / fp16 / fp32, up to 8192 two-byte or 4096 four-byte
@@ -55,7 +55,7 @@ enum tt_norm_status {
 enum tt_norm_dtype {
     TT_NORM_BF16 = 0,
     TT_NORM_F32 = 1,
-    TT_NORM_F16 = 2 /* any-width kernels only */
+    TT_NORM_F16 = 2
 };
 
 /* ABI version of the loaded library (TT_NORM_ABI_VERSION at build time). */
@@ -71,7 +71,7 @@ const char *tt_norm_last_error(void);
  * their workspace queries) accept (cols, dtype), else 0. */
 int tt_norm_supported(int64_t cols, int dtype);
 
-/* 1 if (cols, dtype) is one of the tuned shapes (cols 128 or 3072, bf16 or fp32): the only
+/* 1 if (cols, dtype) is one of the tuned shapes (cols 128 or 3072; bf16, fp16 or fp32): the only
  * ones the reference-contract (*_from_out, *_xnorm, *_from_xnorm) and strided entry points
  * take; the gated residual entry points take cols 3072 only. */
 int tt_norm_tuned(int64_t cols, int dtype);

@@ -157,9 +157,9 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            if constexpr (kIsBf16<T>) {  // row sum straight from the packed pairs
+            if constexpr (kHasDot2<T>) {  // row sum straight from the packed pairs
 #pragma unroll
-                for (int i = 0; i < 4; ++i) s = dot2_bf16(xr[k][i], kBf16OnesPair, s);
+                for (int i = 0; i < 4; ++i) s = dot2<T>(xr[k][i], kOnesPair<T>, s);
             } else {
                 float v[VEC];
                 E::unpack(xr[k], v);
@@ -345,12 +345,12 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
             for (int j = 0; j < VEC; ++j) gv[j] *= tv[k][j];
             gxp[k] = E::pack(gv);  // gx materialised in the element type
-            if constexpr (kIsBf16<T>) {
+            if constexpr (kHasDot2<T>) {
                 // s2 accumulates sum_c gx * xin here; turned into sum_c gx * xhat below
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s1 = dot2_bf16(gxp[k][i], kBf16OnesPair, s1);
-                    s2 = dot2_bf16(gxp[k][i], b.x[k][i], s2);
+                    s1 = dot2<T>(gxp[k][i], kOnesPair<T>, s1);
+                    s2 = dot2<T>(gxp[k][i], b.x[k][i], s2);
                 }
             } else {
                 float gx[VEC], xv[VEC];
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         s1 = group_sum<LANES>(s1);
         s2 = group_sum<LANES>(s2);
         between_passes();
-        if constexpr (kIsBf16<T> && !FROM_XNORM) s2 = r * (s2 - mu * s1);
+        if constexpr (kHasDot2<T> && !FROM_XNORM) s2 = r * (s2 - mu * s1);
         const float m1 = s1 / (float)C, m2 = s2 / (float)C;
         // dx = r*gx + xhat*k1 + k0,  k1 = -r*m2, k0 = -r*m1;  in terms of xin: r*gx + xin*K1 + K0
         const float k1 = -(r * m2), k0 = -(r * m1);
@@ -540,7 +540,7 @@ static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sam
         return fail(TT_NORM_EINVAL, "%s: batch=%lld rows_per_sample=%lld cols=%lld", who, (long long)batch,
                     (long long)rows_per_sample, (long long)cols);
     if (tuned_only && !tuned_shape(cols, dtype))
-        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072, bf16/fp32)", who,
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072)", who,
                     (long long)cols, dtype);
     if (!tt_norm_supported(cols, dtype))
         return fail(TT_NORM_EUNSUPPORTED,
@@ -563,6 +563,9 @@ using namespace ttn;
         if ((dtype) == TT_NORM_BF16) {                           \
             if ((cols) == 128) { CALL(bf16_t, 128); }            \
             else { CALL(bf16_t, 3072); }                         \
+        } else if ((dtype) == TT_NORM_F16) {                     \
+            if ((cols) == 128) { CALL(f16_t, 128); }             \
+            else { CALL(f16_t, 3072); }                          \
         } else {                                                 \
             if ((cols) == 128) { CALL(float, 128); }             \
             else { CALL(float, 3072); }                          \
@@ -663,6 +666,8 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
     const GatedPtrs gp{h2, nullptr, attn, gate};
     if (dtype == TT_NORM_BF16)
         return adaln_forward_t<bf16_t, 3072, false, true>(out, nullptr, mean, rstd, h, scale, shift, a, gp);
+    if (dtype == TT_NORM_F16)
+        return adaln_forward_t<f16_t, 3072, false, true>(out, nullptr, mean, rstd, h, scale, shift, a, gp);
     return adaln_forward_t<float, 3072, false, true>(out, nullptr, mean, rstd, h, scale, shift, a, gp);
 }
 
@@ -690,6 +695,9 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
     if (dtype == TT_NORM_BF16)
         return adaln_backward_t<bf16_t, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
                                                            workspace, workspace_bytes, a, dgate, gp);
+    if (dtype == TT_NORM_F16)
+        return adaln_backward_t<f16_t, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
+                                                          workspace, workspace_bytes, a, dgate, gp);
     return adaln_backward_t<float, 3072, false, true>(dh, dscale, dshift, dout, h2, scale, mean, rstd, dtype,
                                                       workspace, workspace_bytes, a, dgate, gp);
 }
@@ -711,6 +719,9 @@ int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void 
     if (dtype == TT_NORM_BF16)
         return adaln_backward_t<bf16_t, 3072, false, false, true>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype,
                                                                   workspace, workspace_bytes, a, nullptr, gp);
+    if (dtype == TT_NORM_F16)
+        return adaln_backward_t<f16_t, 3072, false, false, true>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype,
+                                                                 workspace, workspace_bytes, a, nullptr, gp);
     return adaln_backward_t<float, 3072, false, false, true>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype,
                                                              workspace, workspace_bytes, a, nullptr, gp);
 }

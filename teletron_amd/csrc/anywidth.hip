@@ -407,12 +407,12 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
             const u32x4 gxk = gx_of(k);
             if constexpr (kKeepGx) gxp[k] = gxk;
             // padding: g = 0 there, so gx = 0 and neither sum sees xhat = nmr
-            if constexpr (kIsBf16<T>) {
+            if constexpr (kHasDot2<T>) {
                 // straight from the packed pairs; s2 holds sum_c gx * x here, turned into sum_c gx * xhat below
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s1 = dot2_bf16(gxk[i], kBf16OnesPair, s1);
-                    s2 = dot2_bf16(gxk[i], xr[k][i], s2);
+                    s1 = dot2<T>(gxk[i], kOnesPair<T>, s1);
+                    s2 = dot2<T>(gxk[i], xr[k][i], s2);
                 }
             } else {
                 float gv[VEC], xv[VEC];
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
         }
         s1 = group_sum<LANES>(s1);
         s2 = group_sum<LANES>(s2);
-        if constexpr (kIsBf16<T>) s2 = r * (s2 - mu * s1);
+        if constexpr (kHasDot2<T>) s2 = r * (s2 - mu * s1);
         const float m1 = s1 / (float)C, m2 = s2 / (float)C;
         // dx = r*(gx - m1 - xhat*m2) = r*gx + x*K1 + K0
         const float k1 = -(r * m2), k0 = -(r * m1);

@@ -56,15 +56,24 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 
 template <typename T>
 inline constexpr bool kIsBf16 = std::is_same<T, bf16_t>::value;
+// 2-byte element types have a packed dot-product instruction.
+template <typename T>
+inline constexpr bool kHasDot2 = sizeof(T) == 2;
 
-constexpr uint32_t kBf16OnesPair = 0x3F803F80u;  // (1.0, 1.0) as two bf16
+// (1.0, 1.0) as two elements of T in one dword.
+template <typename T>
+inline constexpr uint32_t kOnesPair = kIsBf16<T> ? 0x3F803F80u : 0x3C003C00u;
 
-// acc + a.lo*b.lo + a.hi*b.hi over one dword of two bf16 each (v_dot2c_f32_bf16):
-// products of bf16 pairs are exact in fp32, so this is a row reduction step
-// taken straight from the packed registers, with no unpacking.
-__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
-                                           false);
+// acc + a.lo*b.lo + a.hi*b.hi over one dword of two elements each (v_dot2c_f32_bf16 /
+// v_dot2_f32_f16): products of bf16 or fp16 pairs are exact in fp32, so this is a row
+// reduction step taken straight from the packed registers, with no unpacking.
+template <typename T>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    if constexpr (kIsBf16<T>)
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
+                                               false);
+    else
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
 }
 
 template <typename T>

@@ -24,7 +24,7 @@ inline size_t elem_bytes(int dtype) { return dtype == TT_NORM_F32 ? 4 : 2; }
 
 // (cols, dtype) the tuned kernels of rmsnorm.hip / adaln.hip are built for.
 inline bool tuned_shape(int64_t cols, int dtype) {
-    return (cols == 128 || cols == 3072) && (dtype == TT_NORM_BF16 || dtype == TT_NORM_F32);
+    return (cols == 128 || cols == 3072) && (dtype == TT_NORM_BF16 || dtype == TT_NORM_F32 || dtype == TT_NORM_F16);
 }
 
 // Checks the last launch on this thread; returns TT_NORM_OK or TT_NORM_EHIP.

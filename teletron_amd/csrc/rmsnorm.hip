@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
-    constexpr bool kPackedDot = kIsBf16<T> && !FROM_OUT;  // sum_c gy*x straight from bf16 pairs
+    constexpr bool kPackedDot = kHasDot2<T> && !FROM_OUT;  // sum_c gy*x straight from the packed pairs
     // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
     constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_RMS_BWD_ROW_BUFFERS;
     __shared__ float lds[C];
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             gyp[k] = E::pack(gv);  // gy materialised in the element type
             if constexpr (kPackedDot) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) dot = dot2_bf16(gyp[k][i], b.x[k][i], dot);
+                for (int i = 0; i < 4; ++i) dot = dot2<T>(gyp[k][i], b.x[k][i], dot);
             } else {
                 float gy[VEC], xv[VEC];
                 E::unpack(gyp[k], gy);
@@ -361,7 +361,7 @@ static int check_rms_args(const char *who, int64_t rows, int64_t cols, int dtype
                           std::initializer_list<const void *> ptrs, bool tuned_only = false) {
     if (rows < 0 || cols <= 0) return fail(TT_NORM_EINVAL, "%s: rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
     if (tuned_only && !tuned_shape(cols, dtype))
-        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072, bf16/fp32)", who,
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld dtype=%d (this entry point: cols 128/3072)", who,
                     (long long)cols, dtype);
     if (!tt_norm_supported(cols, dtype))
         return fail(TT_NORM_EUNSUPPORTED,
@@ -384,6 +384,9 @@ using namespace ttn;
         if ((dtype) == TT_NORM_BF16) {                           \
             if ((cols) == 128) { CALL(bf16_t, 128); }            \
             else { CALL(bf16_t, 3072); }                         \
+        } else if ((dtype) == TT_NORM_F16) {                     \
+            if ((cols) == 128) { CALL(f16_t, 128); }             \
+            else { CALL(f16_t, 3072); }                          \
         } else {                                                 \
             if ((cols) == 128) { CALL(float, 128); }             \
             else { CALL(float, 3072); }                          \

@@ -15,7 +15,7 @@ What differs from the reference, on purpose:
     back per sample, which is what the eager formula at :223 computes; the
     reference kernels only handle a single modulation row;
   * both operators accept any row of whole 16-byte pieces (up to 8192 two-byte or
-    4096 four-byte columns) in bf16, fp16 or fp32; 128 and 3072 columns in bf16 / fp32
+    4096 four-byte columns) in bf16, fp16 or fp32; 128 and 3072 columns
     run the tuned kernels, and only those take strided views or the gated form;
   * gated_residual_layer_norm fuses the residual update in front of a modulated
     LayerNorm (dit_layerspec.py:152-163) into the norm, forward and backward;
@@ -162,15 +162,15 @@ class AdaLNResidualFunction(Function):
     itself, handed back as an output for the caller to continue the residual stream with
     (dit_layerspec.py:126-131 then :152).  Routing the stream through the Function lets backward add the
     gradient it collected downstream to the norm's dx inside the kernel, in place of the separate
-    accumulation pass autograd runs when a tensor has two consumers.  3072 columns, bfloat16 / float32."""
+    accumulation pass autograd runs when a tensor has two consumers.  3072 columns."""
 
     @staticmethod
     def forward(ctx, x, scale, shift, epsilon):
         ext = _require_extension(fused_adaln, "fused_adaln")
         _require_gpu(x, "AdaLNResidualFunction")
         cols = x.shape[-1]
-        if cols != 3072 or x.dtype not in (torch.bfloat16, torch.float32):
-            raise ValueError(f"AdaLNResidualFunction needs 3072 columns in bfloat16/float32, got {cols}, {x.dtype}")
+        if cols != 3072 or x.dtype not in _ELEM_BYTES:
+            raise ValueError(f"AdaLNResidualFunction needs 3072 columns in bfloat16/float16/float32, got {cols}, {x.dtype}")
         x_c = _aligned_contiguous(x)
         scale_c, shift_c = scale.contiguous().to(x.dtype), shift.contiguous().to(x.dtype)
         if scale_c.numel() % cols or shift_c.numel() != scale_c.numel():
@@ -433,7 +433,7 @@ class RMSNormModelFunction(Function):
             raise ValueError(_unsupported(cols, x.dtype))
         if weight.numel() != cols:
             raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
-        tuned = cols in TUNED_COLS and x.dtype in (torch.bfloat16, torch.float32)
+        tuned = cols in TUNED_COLS and x.dtype in _ELEM_BYTES
         strided = tuned and x.shape[-1] == cols and _strided_rows_ok(x)
         if not strided:
             x = _aligned_contiguous(x)
@@ -500,7 +500,7 @@ class QKVSplitNormFunction(Function):
     Backward writes the gradients of q and k from the kernels directly into their slices of one
     [B, S, H, 3*D] gradient tensor and copies the gradient of v into its slice, so the concatenation
     that torch.split's backward would run over three separate gradients never happens.
-    D must be 128 or 3072, dtype bfloat16 or float32."""
+    D must be 128 or 3072."""
 
     @staticmethod
     def forward(ctx, mixed_qkv, weight_q, weight_k, epsilon):
@@ -509,8 +509,8 @@ class QKVSplitNormFunction(Function):
         if mixed_qkv.dim() != 4 or mixed_qkv.shape[-1] % 3:
             raise ValueError(f"mixed_qkv must be [B, S, H, 3*D], got {tuple(mixed_qkv.shape)}")
         cols = mixed_qkv.shape[-1] // 3
-        if cols not in TUNED_COLS or mixed_qkv.dtype not in (torch.bfloat16, torch.float32):
-            raise ValueError(f"QKVSplitNormFunction needs D in {TUNED_COLS} and bfloat16/float32, got D={cols}, "
+        if cols not in TUNED_COLS or mixed_qkv.dtype not in _ELEM_BYTES:
+            raise ValueError(f"QKVSplitNormFunction needs D in {TUNED_COLS} and bfloat16/float16/float32, got D={cols}, "
                              f"{mixed_qkv.dtype}")
         if weight_q.numel() != cols or weight_k.numel() != cols:
             raise ValueError(f"weights must have {cols} elements")
@@ -565,7 +565,7 @@ def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSN
     FUSED_KERNELS is on and the head dimension is one the tuned kernels take; the reference's own
     sequence of operations otherwise."""
     D = mixed_qkv.shape[-1] // 3
-    if (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in (torch.bfloat16, torch.float32)
+    if (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in _ELEM_BYTES
             and q_norm.eps == k_norm.eps):
         return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
     query, key, value = torch.split(mixed_qkv, [D, D, D], dim=3)

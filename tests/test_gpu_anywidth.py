@@ -105,9 +105,8 @@ def test_adaln_any_width_vs_eager(capi, gpu_device, batch, seq, cols, dtype):
     assert all(torch.equal(a, b) for a, b in zip((dx, ds, dh), again))
 
 
-def test_tuned_and_any_width_kernels_agree_bitwise_on_statistics(capi, gpu_device):
-    """3072 columns in fp16 run the any-width kernels; the same values held in bf16-exact form must give
-    the same row statistics as the tuned bf16 kernels (same sums in the same lane order)."""
+def test_fp16_and_bf16_kernels_agree_on_statistics(capi, gpu_device):
+    """The same values held in fp16 and in bf16 (where both are exact) give the same row statistics."""
     d = O.make_adaln_inputs(2, 131, 3072, BF, seed=7)
     x = d["x"].to(gpu_device)
     sc, sh = d["scale"].to(gpu_device), d["shift"].to(gpu_device)
@@ -195,3 +194,44 @@ def test_geometry_boundaries_forward_and_backward(capi, gpu_device):
         colsum_ok(dh, a_dh, a["grad"].float(), 1, f"adaln dshift cols={cols}")
         xn = torch.nn.functional.layer_norm(a["x"].float(), (cols,), None, None, EPS)
         colsum_ok(ds, a_ds, a["grad"].float() * xn, 1, f"adaln dscale cols={cols}")
+
+
+def test_fp16_through_the_tuned_only_entry_points(capi, gpu_device):
+    """fp16 at 128 / 3072 columns runs the tuned kernels, so the strided, gated and residual forms take it too."""
+    from teletron_amd import fusedlayers as FL
+    # strided QK-norm on the fused projection, forward and backward through the Function
+    B, S, H, D = 1, 203, 6, 128
+    gen = torch.Generator().manual_seed(91)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).half()
+    wq, wk = (1 + 0.02 * torch.randn(D, generator=gen)).half(), (1 + 0.02 * torch.randn(D, generator=gen)).half()
+    gq, gk, gv = (torch.randn(B, H, S, D, generator=gen).half() for _ in range(3))
+    m_c = mixed.clone().requires_grad_(True)
+    q_c, k_c, v_c = torch.split(m_c, [D, D, D], dim=3)
+    q_c, k_c = O.eager_rmsnorm(q_c.transpose(1, 2), wq), O.eager_rmsnorm(k_c.transpose(1, 2), wk)
+    torch.autograd.backward([q_c, k_c, v_c.transpose(1, 2)], [gq, gk, gv])
+    m_g = mixed.to(gpu_device).requires_grad_(True)
+    q_g, k_g, v_g = FL.QKVSplitNormFunction.apply(m_g, wq.to(gpu_device), wk.to(gpu_device), EPS)
+    fwd_16bit_ok(q_g.detach(), q_c.detach(), O.rmsnorm_excuse(q_c.detach()), "q")
+    fwd_16bit_ok(k_g.detach(), k_c.detach(), O.rmsnorm_excuse(k_c.detach()), "k")
+    torch.autograd.backward([q_g, k_g, v_g], [gq.to(gpu_device), gk.to(gpu_device), gv.to(gpu_device)])
+    grad_ok(m_g.grad, m_c.grad, "d mixed")
+    # gated residual + AdaLN
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(2, 257, 3072, HF, seed=92)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    dev_ = lambda t: t.to(gpu_device)
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(dev_(h), dev_(a), dev_(q), dev_(sc), dev_(sh), EPS)
+    assert torch.equal(h2.cpu(), want[0])
+    fwd_16bit_ok(out, want[1], O.adaln_excuse(want[0], sc, sh, want[1]), "gated out")
+    dh, da, dq, dsc, dsh = capi.gated_residual_adaln_backward(dev_(go), dev_(g2), h2, dev_(a), dev_(q), dev_(sc), mean, rstd)
+    terms = want[2].float().abs() + g2.float().abs()
+    assert O.frac_outside(dh.cpu(), want[2], 1e-2, 1e-3, magnitude=terms) <= 1e-4
+    assert O.frac_outside(da.cpu(), want[3], 1e-2, 1e-3, magnitude=terms * q.float().abs()[:, None]) <= 1e-4
+    assert O.colsum_outside(dq.cpu(), want[4], terms * a.float(), dim=1) == 0
+    grad_ok(dsc, want[5], "dscale")
+    grad_ok(dsh, want[6], "dshift")
+    # residual form == plain backward, then the addition
+    x, gr, other = dev_(h), dev_(go), dev_(g2)
+    _, mean, rstd = capi.adaln_forward(x, dev_(sc), dev_(sh), EPS)
+    dx, _, _ = capi.adaln_backward(gr, x, dev_(sc), mean, rstd)
+    dxr, _, _ = capi.adaln_backward_residual(gr, other, x, dev_(sc), mean, rstd)
+    assert torch.equal(dxr, dx + other)

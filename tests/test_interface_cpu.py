@@ -39,9 +39,9 @@ def test_c_abi_exports_every_declared_symbol():
     assert L.tt_norm_supported(8200, capi.BF16) == 0
     # the tuned shapes: the only ones the reference-contract, strided and gated entry points take
     assert L.tt_norm_tuned(3072, capi.BF16) == 1 and L.tt_norm_tuned(128, capi.F32) == 1
-    assert L.tt_norm_tuned(3072, capi.F16) == 0 and L.tt_norm_tuned(256, capi.BF16) == 0
+    assert L.tt_norm_tuned(3072, capi.F16) == 1 and L.tt_norm_tuned(256, capi.BF16) == 0
     assert L.tt_rmsnorm_backward_from_out(None, None, None, None, None, None, 4, 256, 0, None, 0, None) == 2
-    assert L.tt_adaln_forward_xnorm(None, None, None, None, None, None, 1, 4, 3072, 1e-6, capi.F16, None) == 2
+    assert L.tt_adaln_forward_xnorm(None, None, None, None, None, None, 1, 4, 1536, 1e-6, capi.F16, None) == 2
 
 
 def test_c_abi_argument_errors_need_no_gpu():
