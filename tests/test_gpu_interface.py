@@ -416,3 +416,51 @@ def test_empty_and_unaligned_inputs(FL, gpu_device):
     got = FL.RMSNormModelFunction.apply(x_odd, d["weight"].to(gpu_device), EPS, 128)
     want = O.eager_rmsnorm(d["x"], d["weight"], EPS)
     fwd_ok(got, want, O.rmsnorm_excuse(want))
+
+
+def test_block_norm_path_composed_from_the_fused_functions(FL, gpu_device):
+    """The normalisation dataflow of one double-stream block (dit_layerspec.py:126-184) built from the fused
+    Functions -- entry norm keeping the residual stream, QKV split + per-head norms, gated residual + norm2,
+    closing gated update -- against the same graph in eager ops, in fp32 (so that the stand-in GEMMs agree
+    across devices).  Attention and MLP are replaced by cheap differentiable stand-ins."""
+    B, S, H, D = 2, 40, 24, 128
+    C = H * D
+    gen = torch.Generator().manual_seed(123)
+    rnd = lambda *shape, k=1.0: k * torch.randn(*shape, generator=gen)
+    leaves = dict(x=rnd(B, S, C), w_qkv=rnd(C, 3 * C, k=C ** -0.5), wq=1 + rnd(D, k=0.02), wk=1 + rnd(D, k=0.02),
+                  sc1=rnd(B, C, k=0.2), sh1=rnd(B, C, k=0.2), g1=rnd(B, C, k=0.3), sc2=rnd(B, C, k=0.2),
+                  sh2=rnd(B, C, k=0.2), g2=rnd(B, C, k=0.3))
+    g_out = rnd(B, S, C)
+
+    def block(t, fused):
+        x = t["x"]
+        if fused:
+            x_res, n1 = FL.modulated_layer_norm_keeping_stream(x, t["sc1"], t["sh1"], EPS)
+        else:
+            x_res, n1 = x, O.eager_adaln(x, t["sc1"], t["sh1"], EPS)
+        mixed = (n1 @ t["w_qkv"]).view(B, S, H, 3 * D)
+        if fused:
+            q, k, v = FL.QKVSplitNormFunction.apply(mixed, t["wq"], t["wk"], EPS)
+        else:
+            q, k, v = torch.split(mixed, [D, D, D], dim=3)
+            q, k, v = O.eager_rmsnorm(q.transpose(1, 2), t["wq"]), O.eager_rmsnorm(k.transpose(1, 2), t["wk"]), v.transpose(1, 2)
+        attn = (q * torch.sigmoid(k) + v).transpose(1, 2).reshape(B, S, C)          # stand-in for attention + projection
+        if fused:
+            h2, n2 = FL.gated_residual_layer_norm(x_res, attn, t["g1"], t["sc2"], t["sh2"], EPS)
+        else:
+            h2, n2 = O.eager_gated_residual_adaln(x_res, attn, t["g1"], t["sc2"], t["sh2"], EPS)
+        mlp = torch.tanh(n2) * 0.7                                                   # stand-in for the MLP
+        return h2 + t["g2"].unsqueeze(1) * mlp
+
+    cpu = {k: v.clone().requires_grad_(True) for k, v in leaves.items()}
+    gpu = {k: v.to(gpu_device).requires_grad_(True) for k, v in leaves.items()}
+    out_c = block(cpu, fused=False)
+    out_c.backward(g_out)
+    out_g = block(gpu, fused=True)
+    out_g.backward(g_out.to(gpu_device))
+    torch.testing.assert_close(out_g.detach().cpu(), out_c.detach(), rtol=1e-4, atol=1e-4)
+    for name in leaves:
+        want = cpu[name].grad
+        got = gpu[name].grad.cpu()
+        scale = want.abs().max()
+        assert (got - want).abs().max() <= 2e-4 * scale + 1e-5, (name, float((got - want).abs().max()), float(scale))
