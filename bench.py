@@ -61,6 +61,8 @@ WORKLOADS = {
             "forward and backward of the chain (4 C-ABI calls)",
     "w1536-f16": "237600 tokens x 1536 fp16 (a smaller model's hidden size, the any-width kernels); fused RMSNorm "
                  "fwd+bwd + fused AdaLN fwd+bwd per step (4 C-ABI calls)",
+    "cfg4-eager-gpu": "cfg4's step computed by the reference's eager formulas as PyTorch ops on the same GPU "
+                      "(what the reference runs with FUSED_KERNELS off): a baseline, not this library",
     "qkv-site": "the QK-norm call site through the autograd Function: [1, 29700, 24, 384] bf16 fused projection -> "
                 "q, k normalised [B, H, S, 128] + v view, forward + backward with the projection's gradient "
                 "assembled in place (QKVSplitNormFunction); traffic counted as 12 slice-sized tensors",
@@ -172,6 +174,24 @@ def build_workload(name, torch, capi, dev):
         # chain order: AdaLN fwd, RMSNorm fwd, RMSNorm bwd, AdaLN bwd (the gradient buffers are stand-ins of the
         # right size: timing does not depend on their values)
         return [ada[0], rms[0], rms[1], ada[1]], B * S * COLS * 2, B * S, "bf16", x
+    if name == "cfg4-eager-gpu":
+        x = rnd(1, ROWS, COLS, dtype=bf).requires_grad_(True)
+        grad = rnd(1, ROWS, COLS, dtype=bf)
+        w = rnd(COLS, dtype=bf, k=0.02, bias=1.0).requires_grad_(True)
+        scale, shift = (rnd(1, COLS, dtype=bf, k=0.1).requires_grad_(True) for _ in range(2))
+
+        def eager_rmsnorm():     # teletron/models/dit/dit_fusedlayers.py:360-370
+            y = (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + EPS)).type_as(x) * w
+            y.backward(grad)
+            x.grad = None
+
+        def eager_adaln():       # teletron/models/dit/dit_fusedlayers.py:198,223
+            y = torch.nn.functional.layer_norm(x, (COLS,), None, None, EPS) * (1 + scale[:, None]) + shift[:, None]
+            y.backward(grad)
+            x.grad = None
+
+        return [("eager_rmsnorm_fwd_bwd", eager_rmsnorm, 5), ("eager_adaln_fwd_bwd", eager_adaln, 5)], \
+            ROWS * COLS * 2, 2 * ROWS, "bf16", grad
     if name in ("qkv-site", "qkv-site-reference"):
         from teletron_amd import fusedlayers as FL
         B, S, H, D = 1, 29700, 24, 128
@@ -342,7 +362,7 @@ def main():
         return e
 
     # a call that is a whole autograd forward + backward launches several row kernels: no single one to bracket
-    composite = args.workload.startswith("qkv-site")
+    composite = args.workload.startswith("qkv-site") or args.workload == "cfg4-eager-gpu"
     pairs = [] if (args.hip_graph or composite) else [(hip_event(), hip_event()) for _ in range(args.steps)]
     arm = L.tt_norm_profile_next_row_kernel
     graphs = []
