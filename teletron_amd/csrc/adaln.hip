@@ -34,7 +34,7 @@
 #ifndef TTN_ADALN_BWD_PREFETCH_MID
 #define TTN_ADALN_BWD_PREFETCH_MID 1
 #endif
-// Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
+// Stores of dx / out: 1 = write-through at device scope (RowWriter<1>), 0 = plain streaming store.
 // Backward (2 reads + 1 write): 379 -> 358 us with write-through; the gated backward (4 reads + 2 writes)
 // and the forward kernels measure the same either way and stay plain.
 #ifndef TTN_ADALN_FWD_STORE
@@ -128,13 +128,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         const bool ok = rs < rows_per_sample;
         const int64_t row = b * rows_per_sample + rs;
+        // the wavefront's rows are consecutive: where it writes starts at its first row
+        const int64_t first = (b * rows_per_sample + grp * RPW) * C;
+        const uint32_t lane_bytes = (uint32_t)((sub * C) * sizeof(T)) + l * 16;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(x + row * C) + l;
         u32x4 xr[CHUNKS];
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
         if constexpr (GATED) {
             const u32x4 *pa = reinterpret_cast<const u32x4 *>(attn + row * C) + l;
-            u32x4 *ph = reinterpret_cast<u32x4 *>(h2_out + row * C) + l;
+            const RowWriter<TTN_ADALN_FWD_STORE> wh(h2_out + first, lane_bytes);
             u32x4 ar[CHUNKS];
 #pragma unroll
             for (int k = 0; k < CHUNKS; ++k) ar[k] = ok ? load16_stream(pa + k * LANES) : u32x4{0, 0, 0, 0};
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) hv[j] += av[j];
                 xr[k] = E::pack(hv);  // h2: the new residual stream, and the row that is normalised
-                if (ok) store16<TTN_ADALN_FWD_STORE>(ph + k * LANES, xr[k]);
+                if (ok) wh.put(k * LANES, xr[k]);
             }
         }
 
@@ -186,8 +189,8 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         }
 
         const float nmr = -(mu * r);
-        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
-        u32x4 *pn = WRITE_XNORM ? reinterpret_cast<u32x4 *>(xnorm + row * C) + l : nullptr;
+        const RowWriter<TTN_ADALN_FWD_STORE> wo(out + first, lane_bytes);
+        const RowWriter<TTN_ADALN_FWD_STORE> wn(WRITE_XNORM ? xnorm + first : nullptr, lane_bytes);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], tv[VEC], hv[VEC];
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r as x*r + (-mu*r)
             if constexpr (WRITE_XNORM) {
                 const u32x4 xn = E::pack(v);
-                if (ok) store16<TTN_ADALN_FWD_STORE>(pn + k * LANES, xn);
+                if (ok) wn.put(k * LANES, xn);
                 E::unpack(xn, v);
             } else {
                 E::round(v);  // xn
@@ -208,7 +211,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::round(v);  // xn * (1 + scale)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] += hv[j];
-            if (ok) store16<TTN_ADALN_FWD_STORE>(po + k * LANES, E::pack(v));
+            if (ok) wo.put(k * LANES, E::pack(v));
         }
     }
 }
@@ -244,6 +247,9 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
     // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
     constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_ADALN_BWD_ROW_BUFFERS;
+    // A row's first pass starts only when the stores of the row before it have left the wavefront
+    // (see the RMSNorm backward): 359 us with this wait, 366 us without, at 118 800 rows.
+    constexpr bool kDrainStores = TTN_ADALN_BWD_STORE && !GATED && kRowBuffers == 2 && C >= 1024;
     __shared__ float lds[NSETS * C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
@@ -285,12 +291,14 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         u32x4 a[kEarlyOperands ? CHUNKS : 1], e[(kEarlyOperands || RES) ? CHUNKS : 1];
         float r, mu;
         int64_t row;
+        int64_t first;  // element offset of the wavefront's first row (wave-uniform)
         bool ok;
     };
     auto fetch = [&](RowRegs &b, int64_t grp) {
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         b.ok = rs < rows_per_sample;
         b.row = smp * rows_per_sample + rs;
+        b.first = (smp * rows_per_sample + grp * RPW) * C;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
 #if TTN_BWD_LOAD_RUNS
@@ -338,6 +346,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         // pass 1: gx = rnd(g*t) kept packed; s1 = sum_c gx; s2 = sum_c gx * xhat
         u32x4 gxp[CHUNKS];
         float s1 = 0.0f, s2 = 0.0f;
+        if constexpr (kDrainStores) wait_memory_ops<0>();
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC];
@@ -373,7 +382,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         const float K1 = FROM_XNORM ? k1 : k1 * r;
         const float K0 = FROM_XNORM ? k0 : fmaf(k1, nmr, k0);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.row * C) + l;
+        const uint32_t lane_bytes = (uint32_t)((sub * C) * sizeof(T)) + l * 16;
+        constexpr int kDxStore = (GATED ? 0 : TTN_ADALN_BWD_STORE);
+        const RowWriter<kDxStore> wd(dx + b.first, lane_bytes);
+        const RowWriter<0> wa(GATED ? da + b.first : nullptr, lane_bytes);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
@@ -404,7 +416,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o[j] += ev[j];
                 const u32x4 dhp = E::pack(o);  // dh: gradient of h2 = of the residual input
-                if (b.ok) store16<0>(pd + k * LANES, dhp);
+                if (b.ok) wd.put(k * LANES, dhp);
                 E::unpack(dhp, o);
                 if constexpr (kGateResident) {
 #pragma unroll
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) av[j] *= o[j];
-                if (b.ok) store16<0>(reinterpret_cast<u32x4 *>(da + b.row * C) + l + k * LANES, E::pack(dav));
+                if (b.ok) wa.put(k * LANES, E::pack(dav));
                 E::round(av);  // dh*attn materialised in the element type before the column sum
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
@@ -428,7 +440,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) o[j] += ev[j];
                 }
-                if (b.ok) store16<TTN_ADALN_BWD_STORE>(pd + k * LANES, E::pack(o));
+                if (b.ok) wd.put(k * LANES, E::pack(o));
             }
             if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
 #pragma unroll

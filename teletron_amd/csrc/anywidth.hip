@@ -16,7 +16,7 @@
 #include "norm_device.h"
 #include "norm_host.h"
 
-// Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
+// Stores of dx / out: 1 = write-through at device scope (RowWriter<1>), 0 = plain streaming store.
 // Measured both ways per width: backward gains up to 7 % with write-through for rows of up to six
 // accesses per lane (512 columns 212 -> 197 us, 1024 196 -> 186 us, 1536 184 -> 182 us) and loses 3-4 %
 // at eight and twelve (4096, 6144 columns), so the wide geometries keep the plain store.
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
         const float r = 1.0f / sqrtf(ss / (float)C + eps);
         if (ok && l == 0) rstd[row] = r;
 
-        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+        const RowWriter<TTN_ANY_FWD_STORE> wo(out + grp * RPW * C, (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], wv[VEC];
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
             E::round(v);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
-            if (ok && m.in[k]) store16<TTN_ANY_FWD_STORE>(po + k * LANES, E::pack(v));
+            if (ok && m.in[k]) wo.put(k * LANES, E::pack(v));
         }
     }
 }
@@ -211,7 +211,8 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
         keep_packed(xr);
         keep_packed(gyp);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+        const RowWriter<(TTN_ANY_BWD_STORE && CHUNKS <= 6)> wd(dx + grp * RPW * C,
+                                                               (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
                 o[j] = fmaf(xv[j], coef, gy[j] * r);
                 y[j] = xv[j] * r;
             }
-            if (ok && m.in[k]) store16<(TTN_ANY_BWD_STORE && CHUNKS <= 6)>(pd + k * LANES, E::pack(o));
+            if (ok && m.in[k]) wd.put(k * LANES, E::pack(o));
             E::round(y);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
@@ -305,7 +306,8 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
         }
 
         const float nmr = -(mu * r);
-        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+        const RowWriter<TTN_ANY_FWD_STORE> wo(out + (b * rows_per_sample + grp * RPW) * C,
+                                              (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], tv[VEC], hv[VEC];
@@ -320,7 +322,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
             E::round(v);  // xn * (1 + scale)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] += hv[j];
-            if (ok && m.in[k]) store16<TTN_ANY_FWD_STORE>(po + k * LANES, E::pack(v));
+            if (ok && m.in[k]) wo.put(k * LANES, E::pack(v));
         }
     }
 }
@@ -438,7 +440,8 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
         keep_packed(xr);
         if constexpr (kKeepGx) keep_packed(gxp);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + row * C) + l;
+        const RowWriter<(TTN_ANY_BWD_STORE && CHUNKS <= 6)> wd(dx + (b * rows_per_sample + grp * RPW) * C,
+                                                               (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
                 xn[j] = fmaf(xv[j], r, nmr);
                 acc[1][k][j] += gv[j];
             }
-            if (ok && m.in[k]) store16<(TTN_ANY_BWD_STORE && CHUNKS <= 6)>(pd + k * LANES, E::pack(o));
+            if (ok && m.in[k]) wd.put(k * LANES, E::pack(o));
             E::round(xn);  // the normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];

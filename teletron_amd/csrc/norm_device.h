@@ -163,24 +163,56 @@ struct RowGeom {
 // they carry the non-temporal hint; parameters use the plain cached forms.
 __device__ __forceinline__ u32x4 load16_stream(const u32x4 *p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void store16_stream(u32x4 *p, const u32x4 &v) { __builtin_nontemporal_store(v, p); }
-// The same store marked write-through at device scope (sc1) as well as non-temporal: the line goes to
-// memory as it is written instead of waiting dirty in L2 for an eviction.  Written as an instruction
-// so that the stores of a row are issued where the source puts them.  Measured on the backward
-// kernels (2 reads + 1 write): 367 -> 354 us; no gain on 1 read + 1 write.
-// The s_nop is required: a store of more than 8 bytes reads its data registers one cycle after it
-// issues, and the compiler, which cannot see what the asm is, may overwrite them in the very next
-// instruction (it inserts this wait state itself after the stores it generates).
-__device__ __forceinline__ void store16_through(u32x4 *p, const u32x4 &v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" ::"v"(p), "v"(v));
-}
-template <int THROUGH>
-__device__ __forceinline__ void store16(u32x4 *p, const u32x4 &v) {
-    if constexpr (THROUGH)
-        store16_through(p, v);
-    else
-        store16_stream(p, v);
-}
 __device__ __forceinline__ u32x4 load16(const u32x4 *p) { return *p; }
+
+// Where a wavefront writes the rows of one loop iteration: a wave-uniform base address (the first of
+// the wavefront's rows) plus a per-lane byte offset below 2 GiB; put(piece, v) stores 16 bytes at
+// 16-byte piece `piece` (a compile-time multiple of LANES) past the lane's position.
+//   THROUGH = 0: plain streaming store (non-temporal hint).
+//   THROUGH = 1: the same store marked write-through at device scope (sc1) as well as non-temporal:
+//     the line goes to memory as it is written instead of waiting dirty in L2 for an eviction.
+//     Measured on the backward kernels (2 reads + 1 write): 367 -> 354 us; no gain on 1 read +
+//     1 write.  Issued as a buffer store, the one store form whose cache-policy bits the compiler
+//     exposes, so the compiler sees a store: it keeps the wait states after it and counts it in the
+//     memory-operation counter, and a wait for the NEXT row's loads (requested before these stores)
+//     does not wait for these stores as well.
+template <int THROUGH>
+struct RowWriter;
+
+template <>
+struct RowWriter<0> {
+    u32x4 *p;
+    __device__ __forceinline__ RowWriter(void *wave_base, uint32_t lane_bytes)
+        : p(reinterpret_cast<u32x4 *>(static_cast<char *>(wave_base) + lane_bytes)) {}
+    __device__ __forceinline__ void put(int piece, const u32x4 &v) const { store16_stream(p + piece, v); }
+};
+
+template <>
+struct RowWriter<1> {
+    static constexpr uint32_t kRawDwords = 0x00020000u;  // word 3 of a raw (untyped, unswizzled) resource
+    static constexpr int kSc1Nt = 16 | 2;                // cache policy: sc1 (bit 4) | nt (bit 1)
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t off;
+    __device__ __forceinline__ RowWriter(void *wave_base, uint32_t lane_bytes) : off(lane_bytes) {
+        // the base lives in scalar registers; every caller passes a wave-uniform address
+        const uint64_t a = reinterpret_cast<uint64_t>(wave_base);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(((uint64_t)hi << 32) | lo), 0, 0xffffffffu,
+                                                 kRawDwords);
+    }
+    __device__ __forceinline__ void put(int piece, const u32x4 &v) const {
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, piece * 16, kSc1Nt);
+    }
+};
+
+// Waits until at most N of this wavefront's vector-memory operations (loads and stores, which
+// complete in issue order) are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_memory_ops() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
 
 // Makes the compiler forget what it knows about a packed register array (no
 // instruction is emitted).  Used on loop-invariant packed parameters at the

@@ -37,7 +37,7 @@
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
-// Stores of dx / out: 1 = write-through at device scope (store16_through), 0 = plain streaming store.
+// Stores of dx / out: 1 = write-through at device scope (RowWriter<1>), 0 = plain streaming store.
 // Backward (2 reads + 1 write): 367 -> 353 us with write-through.  Forward (1 read + 1 write): the same
 // either way at 3072 columns (one-shot grid), 62.6 -> 61.4 us at 128 columns (persistent grid).
 #ifndef TTN_RMS_FWD_STORE
@@ -146,7 +146,9 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         const float r = 1.0f / sqrtf(ss / (float)C + eps);
         if (ok && l == 0) rstd[row] = r;
 
-        u32x4 *po = reinterpret_cast<u32x4 *>(out + row * C) + l;
+        // the wavefront's rows are consecutive in out: base = its first row
+        const int64_t row0 = map.template locate<RPW, C>(grp, 0).row;
+        const RowWriter<TTN_RMS_FWD_STORE> wo(out + row0 * C, (uint32_t)((sub * C) * sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], wv[VEC];
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::round(v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
-            if (ok) store16<TTN_RMS_FWD_STORE>(po + k * LANES, E::pack(v));
+            if (ok) wo.put(k * LANES, E::pack(v));
         }
     }
 }
@@ -182,6 +184,11 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     constexpr bool kPackedDot = kHasDot2<T> && !FROM_OUT;  // sum_c gy*x straight from the packed pairs
     // row buffers in flight per wavefront; fp32 rows of 3072 take 96 registers each: one only
     constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_RMS_BWD_ROW_BUFFERS;
+    // With the next row requested between the passes, a row's first pass starts only when the stores
+    // of the row before it have left the wavefront (and with them this row's loads, which are older):
+    // one wavefront never has more than one row of loads plus one row of stores outstanding.  Measured
+    // at 118 800 rows: 354 us with this wait, 365 us when the first pass waits for its loads alone.
+    constexpr bool kDrainStores = TTN_RMS_BWD_STORE && kRowBuffers == 2 && C >= 1024;
     __shared__ float lds[C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
@@ -208,13 +215,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     struct RowRegs {
         u32x4 g[CHUNKS], x[CHUNKS];
         float r;
-        int64_t doff;
+        int64_t doff0;   // element offset in dx of the wavefront's first row (wave-uniform)
+        uint32_t dlane;  // this lane's byte offset from there
         bool ok;
     };
     auto fetch = [&](RowRegs &b, int64_t grp) {
         const RowAddr at = map.template locate<RPW, C>(grp, sub);
         b.ok = at.ok;
-        b.doff = at.doff;
+        b.doff0 = map.template locate<RPW, C>(grp, 0).doff;
+        b.dlane = (uint32_t)((at.doff - b.doff0) * (int64_t)sizeof(T)) + l * 16;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
 #if TTN_BWD_LOAD_RUNS
@@ -237,6 +246,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         //   xs = x (native) or xhat = out / w (from the saved output)
         u32x4 gyp[CHUNKS];
         float dot = 0.0f;
+        if constexpr (kDrainStores) wait_memory_ops<0>();
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC];
@@ -260,7 +270,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         // dx = gy*r + xs*coef
         const float coef = FROM_OUT ? -(r * (dot / (float)C)) : -((dot / (float)C) * r * r * r);
 
-        u32x4 *pd = reinterpret_cast<u32x4 *>(dx + b.doff) + l;
+        const RowWriter<TTN_RMS_BWD_STORE> wd(dx + b.doff0, b.dlane);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
@@ -273,7 +283,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 o[j] = fmaf(xs, coef, gy[j] * r);
                 y[j] = FROM_OUT ? xs : xs * r;
             }
-            if (b.ok) store16<TTN_RMS_BWD_STORE>(pd + k * LANES, E::pack(o));
+            if (b.ok) wd.put(k * LANES, E::pack(o));
             E::round(y);  // y = normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
@@ -452,11 +462,16 @@ static int check_strided(const char *who, int64_t n0, int64_t n1, int64_t n2, in
     if (n0 < 0 || n1 < 0 || n2 < 0)
         return fail(TT_NORM_EINVAL, "%s: sizes [%lld, %lld, %lld]", who, (long long)n0, (long long)n1, (long long)n2);
     if (!tt_norm_supported(cols, dtype)) return TT_NORM_OK;  // reported by the common check
-    const int64_t vec = dtype == TT_NORM_BF16 ? 8 : 4;
+    const int64_t vec = 16 / (int64_t)elem_bytes(dtype);
     for (int64_t s : strides)
         if (s < 0 || s % vec != 0)
             return fail(TT_NORM_EALIGN, "%s: %s stride %lld is not a non-negative multiple of %lld elements (16 bytes)",
                         who, what, (long long)s, (long long)vec);
+    // the rows one wavefront handles together (up to four consecutive indices of the last dimension)
+    // are addressed with 32-bit byte offsets from the first of them
+    if (strides[2] > (int64_t)(1 << 28) / (int64_t)elem_bytes(dtype))
+        return fail(TT_NORM_EINVAL, "%s: %s stride %lld of the row dimension exceeds 256 MiB", who, what,
+                    (long long)strides[2]);
     return TT_NORM_OK;
 }
 

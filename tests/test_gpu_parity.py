@@ -562,6 +562,34 @@ def test_rmsnorm_strided_rejects_unaligned_strides(capi, gpu_device):
     assert e.value.status == 3
 
 
+@pytest.mark.parametrize("dtype,code", [(torch.float16, 2), (torch.bfloat16, 0), (torch.float32, 1)])
+def test_strided_entry_points_reject_strides_that_are_not_16_bytes(capi, gpu_device, dtype, code):
+    """The header promises TT_NORM_EALIGN for strides that are not multiples of 16 bytes, for every
+    element type; checked on the C ABI itself (the Python wrapper has a check of its own in front).
+    The rejection happens on the host: no kernel runs."""
+    L = capi.lib()
+    D, esz = 128, torch.empty(0, dtype=dtype).element_size()
+    half = 8 // esz                                  # elements in 8 bytes: aligned to 8 bytes, not to 16
+    n0, n1, n2 = 2, 3, 5
+    x = torch.zeros(n0 * n1 * n2 * (D + half) + 64, dtype=dtype, device=gpu_device)
+    out = torch.zeros(n0 * n1 * n2 * D, dtype=dtype, device=gpu_device)
+    w = torch.ones(D, dtype=dtype, device=gpu_device)
+    rstd = torch.zeros(n0 * n1 * n2, dtype=torch.float32, device=gpu_device)
+    dw = torch.zeros(D, dtype=dtype, device=gpu_device)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=gpu_device)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    bad = D + half                                   # row stride of D elements + 8 bytes
+    st = L.tt_rmsnorm_forward_strided(p(out), p(rstd), p(x), p(w), n0, n1, n2, n1 * n2 * bad, n2 * bad, bad, D,
+                                      EPS, code, None)
+    assert st == 3, (st, L.tt_norm_last_error())
+    for xs2, ds2 in ((bad, D), (D, bad)):            # the check covers x's strides and dx's strides
+        st = L.tt_rmsnorm_backward_strided(p(out), p(dw), p(out), p(x), p(w), p(rstd), n0, n1, n2,
+                                           n1 * n2 * xs2, n2 * xs2, xs2, n1 * n2 * ds2, n2 * ds2, ds2, D, code,
+                                           p(ws), ws.numel(), None)
+        assert st == 3, (st, L.tt_norm_last_error())
+    torch.cuda.synchronize()
+
+
 def test_profile_hook_brackets_the_row_kernel(capi, gpu_device):
     """tt_norm_profile_next_row_kernel: one shot, records on the launch stream around the row kernel."""
     hip = ctypes.CDLL("libamdhip64.so")
