@@ -69,6 +69,9 @@ WORKLOADS = {
     "qkv-site-reference": "the same call site the reference's way with these kernels: torch.split, transpose, "
                           "contiguous copy, dense RMSNorm Function per tensor, torch.split's backward; same "
                           "traffic accounting as qkv-site (12 slice-sized tensors of useful work)",
+    "stream-ceiling": "plain streams over 729.9 MB tensors: 0-2 tensors read, 0-1 written, 1/2/6 KiB per wavefront per "
+                      "tensor, one-shot and persistent grids, streaming and write-through stores; plus the runtime's "
+                      "and PyTorch's copies (no normalization arithmetic: the bandwidth envelope the kernels live in)",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -236,6 +239,70 @@ def build_workload(name, torch, capi, dev):
     raise ValueError(name)
 
 
+def stream_ceiling(args, torch, capi, dev):
+    """What the memory system gives plain streams of each read/write mix and access shape (library probe
+    kernels over cfg4-sized tensors), next to two copies not written here: the runtime's device-to-device
+    copy and a PyTorch elementwise copy.  Every figure is back-to-back launches between two events."""
+    L = capi.lib()
+    nbytes = ROWS * COLS * 2
+    a = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    b = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    d = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def timed(fn, n_streams):
+        for _ in range(max(3, args.warmup // 4)):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / args.steps * 1e3
+        return {"us": round(us, 1), "GB/s": round(n_streams * nbytes / us / 1e3, 1),
+                "frac_of_peak": round(n_streams * nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    def probe(reads, writes, per_lane, blocks, through):
+        def fn():
+            st = L.tt_norm_stream_probe(p(d), p(a), p(b), nbytes, reads, writes, per_lane, blocks, through, stream)
+            if st != 0:
+                raise RuntimeError(L.tt_norm_last_error().decode())
+        return timed(fn, reads + writes)
+
+    rows = []
+    for reads, writes in ((1, 0), (2, 0), (0, 1), (1, 1), (2, 1)):
+        for per_lane in (1, 2, 6):
+            for blocks in (0, 256, 1024):
+                for through in ((0, 1) if writes and per_lane == 6 else (0,)):
+                    r = probe(reads, writes, per_lane, blocks, through)
+                    r.update({"reads": reads, "writes": writes, "KiB_per_wavefront_per_tensor": per_lane,
+                              "grid": "one-shot" if blocks == 0 else f"persistent {blocks} workgroups",
+                              "store": "write-through" if through else ("streaming" if writes else "-")})
+                    rows.append(r)
+    others = {
+        "hipMemcpyDtoDAsync": timed(lambda: hip.hipMemcpyDtoDAsync(p(d), p(a), ctypes.c_size_t(nbytes), stream), 2),
+        "torch copy_ (bf16)": timed(lambda: d.view(torch.bfloat16).copy_(a.view(torch.bfloat16)), 2),
+        "torch zero_ (write only)": timed(lambda: d.view(torch.bfloat16).zero_(), 1),
+        "tt_norm_stream_copy": timed(lambda: capi.stream_copy(d, a), 2),
+    }
+    best = lambda r_, w_: max((r for r in rows if r["reads"] == r_ and r["writes"] == w_), key=lambda r: r["GB/s"])
+    two_one = best(2, 1)
+    print(json.dumps({
+        "metric": "plain-stream HBM GB/s per read/write mix (ceiling probe), 729.9 MB per tensor",
+        "value": two_one["GB/s"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(two_one["us"] / 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": WORKLOADS["stream-ceiling"], "tensor_bytes": nbytes},
+        "best": {"read_only": best(1, 0), "two_reads": best(2, 0), "write_only": best(0, 1),
+                 "copy_1R_1W": best(1, 1), "2R_1W": two_one},
+        "probes": rows, "other_copies": others,
+    }))
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -298,6 +365,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L = capi.lib()
+    if args.workload == "stream-ceiling":
+        stream_ceiling(args, torch, capi, dev)
+        return
     calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)
     headline = args.workload == "cfg4"
     # A step streams every tensor once.  When a tensor is smaller than twice the 256 MB last-level

@@ -227,6 +227,17 @@ int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event);
  * yardstick the benchmark prints next to each result. */
 int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
 
+/* Measurement only (no counterpart in the reference): a plain stream of `reads` tensors read (0..2: a,
+ * then b) and `writes` tensors written (0..1: dst), `bytes` each, where every wavefront moves one
+ * contiguous run of accesses_per_lane KiB per tensor (1, 2 or 6 accesses of 16 bytes per lane; 6 is
+ * the shape of a 3072-column two-byte row).  persistent_blocks = 0 launches one wavefront per run
+ * (one-shot grid), otherwise that many workgroups of four wavefronts stride over the runs.
+ * write_through != 0 uses the write-through store of the backward kernels.  The benchmark uses it
+ * to print what the memory system gives each read/write mix next to the kernels' own figures.
+ * The event pair armed by tt_norm_profile_next_row_kernel brackets this kernel as well. */
+int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
+                         int accesses_per_lane, int persistent_blocks, int write_through, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,7 @@ EXPORTS = (
     "tt_norm_profile_next_row_kernel",
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
     "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual",
+    "tt_norm_stream_probe",
 )
 
 
@@ -70,6 +71,7 @@ def lib() -> ctypes.CDLL:
         L.tt_gated_residual_adaln_backward.argtypes = [vp] * 13 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_residual.argtypes = [vp] * 9 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
+        L.tt_norm_stream_probe.argtypes = [vp, vp, vp, sz, ci, ci, ci, ci, ci, vp]
         L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
     return _lib

@@ -176,6 +176,54 @@ __global__ __launch_bounds__(kRowThreads) void stream_copy_kernel(u32x4 *__restr
     }
 }
 
+// ---- streaming probe -----------------------------------------------------------
+// Plain streams with the access shapes the row kernels can choose from, for measuring what this
+// memory system gives each read/write mix: NR tensors read (0, 1 or 2), NW written (0 or 1);
+// every wavefront moves one contiguous run of D KiB per tensor (D 16-byte accesses per lane; 6 is
+// a 3072-column two-byte row) and either exits (one-shot grid) or strides on (persistent grid).
+// Loads carry the non-temporal hint; THROUGH picks the store (see RowWriter).
+template <int NR, int NW, int D, int THROUGH>
+__global__ __launch_bounds__(kRowThreads) void stream_probe_kernel(u32x4 *__restrict__ dst,
+                                                                   const u32x4 *__restrict__ a,
+                                                                   const u32x4 *__restrict__ b, int64_t runs,
+                                                                   u32x4 *__restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    u32x4 keep{0, 0, 0, 0};
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t run = (int64_t)blockIdx.x * kRowWaves + wave_id_in_block(); run < runs; run += stride) {
+        const int64_t at = run * (D * kWaveSize);
+        u32x4 v[D];
+#pragma unroll
+        for (int k = 0; k < D; ++k) v[k] = NR >= 1 ? load16_stream(a + at + lane + k * kWaveSize) : u32x4{(uint32_t)run, 1, 2, 3};
+        if constexpr (NR >= 2) {
+            u32x4 w[D];
+#pragma unroll
+            for (int k = 0; k < D; ++k) w[k] = load16_stream(b + at + lane + k * kWaveSize);
+#pragma unroll
+            for (int k = 0; k < D; ++k) v[k] += w[k];
+        }
+        if constexpr (NW >= 1) {
+            const RowWriter<THROUGH> wr(dst + at, lane * 16);
+#pragma unroll
+            for (int k = 0; k < D; ++k) wr.put(k * kWaveSize, v[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < D; ++k) keep += v[k];
+        }
+    }
+    // read-only probes: keep the loads alive without ever storing
+    if (NW == 0 && keep[0] == 0x12345678u && keep[1] == 0x9abcdef0u && keep[2] == 0x0fedcba9u) *sink = keep;
+}
+
+template <int NR, int NW, int D, int THROUGH>
+static int launch_stream_probe(void *dst, const void *a, const void *b, int64_t runs, int64_t blocks,
+                               hipStream_t stream) {
+    RowKernelProfile prof(stream);
+    stream_probe_kernel<NR, NW, D, THROUGH><<<dim3((unsigned)blocks), dim3(kRowThreads), 0, stream>>>(
+        (u32x4 *)dst, (const u32x4 *)a, (const u32x4 *)b, runs, (u32x4 *)dst);
+    return TT_NORM_OK;
+}
+
 }  // namespace ttn
 
 using namespace ttn;
@@ -224,6 +272,37 @@ int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) 
     stream_copy_kernel<<<dim3((unsigned)blocks), dim3(kRowThreads), 0, (hipStream_t)stream>>>(
         (u32x4 *)dst, (const u32x4 *)src, n16);
     return check_launch("stream copy launch");
+}
+
+int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
+                         int accesses_per_lane, int persistent_blocks, int write_through, void *stream) {
+    if (reads < 0 || reads > 2 || writes < 0 || writes > 1 || reads + writes == 0)
+        return fail(TT_NORM_EINVAL, "stream_probe: reads=%d (0..2) writes=%d (0..1), at least one stream", reads, writes);
+    if (accesses_per_lane != 1 && accesses_per_lane != 2 && accesses_per_lane != 6)
+        return fail(TT_NORM_EUNSUPPORTED, "stream_probe: accesses_per_lane=%d (built for 1, 2 and 6)", accesses_per_lane);
+    if (persistent_blocks < 0) return fail(TT_NORM_EINVAL, "stream_probe: persistent_blocks=%d", persistent_blocks);
+    const size_t run_bytes = (size_t)accesses_per_lane * kWaveSize * 16;
+    if (bytes == 0 || bytes % run_bytes)
+        return fail(TT_NORM_EINVAL, "stream_probe: bytes (%zu) must be a positive multiple of %zu", bytes, run_bytes);
+    if (!dst || (reads >= 1 && !a) || (reads >= 2 && !b)) return fail(TT_NORM_EINVAL, "stream_probe: null pointer");
+    if (!aligned16(dst) || !aligned16(a) || !aligned16(b)) return fail(TT_NORM_EALIGN, "stream_probe: unaligned pointer");
+    const int64_t runs = (int64_t)(bytes / run_bytes);
+    const int64_t blocks = persistent_blocks ? persistent_blocks : (runs + kRowWaves - 1) / kRowWaves;
+    if (blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "stream_probe: grid too large");
+    const hipStream_t s = (hipStream_t)stream;
+    const int through = (write_through && writes) ? 1 : 0;
+#define TTN_PROBE(NR, NW, D, TH)                                                          \
+    if (reads == NR && writes == NW && accesses_per_lane == D && through == TH) {         \
+        launch_stream_probe<NR, NW, D, TH>(dst, a, b, runs, blocks, s);                   \
+        return check_launch("stream probe launch");                                       \
+    }
+#define TTN_PROBE_D(NR, NW, TH) TTN_PROBE(NR, NW, 1, TH) TTN_PROBE(NR, NW, 2, TH) TTN_PROBE(NR, NW, 6, TH)
+    TTN_PROBE_D(1, 0, 0) TTN_PROBE_D(2, 0, 0)
+    TTN_PROBE_D(0, 1, 0) TTN_PROBE_D(1, 1, 0) TTN_PROBE_D(2, 1, 0)
+    TTN_PROBE_D(0, 1, 1) TTN_PROBE_D(1, 1, 1) TTN_PROBE_D(2, 1, 1)
+#undef TTN_PROBE_D
+#undef TTN_PROBE
+    return fail(TT_NORM_EUNSUPPORTED, "stream_probe: no kernel for this combination");
 }
 
 }  // extern "C"
