@@ -162,6 +162,21 @@ int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, co
                       int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                       void *workspace, size_t workspace_bytes, void *stream);
 
+/* tt_adaln_backward without a scratch argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The partial column sums go to a static device array of
+ * TT_NORM_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends); the call allocates and frees nothing.  Shapes whose scratch need
+ * (tt_adaln_backward_workspace_bytes) exceeds the array return TT_NORM_EWORKSPACE: at 3072
+ * columns that is batch > 682; every supported width fits for batch <= 256.  Results are
+ * bit-identical to tt_adaln_backward.  All calls on one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (different streams or threads) race; on one stream they are safe. */
+#define TT_NORM_STATIC_SCRATCH_BYTES (16u << 20)
+int tt_adaln_backward_static(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                             const void *scale, const float *mean, const float *rstd,
+                             int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                             void *stream);
+
 /* Same contract as the reference's launch_adaln_backward (adaln_kernel.h:36-45):
  * works from the saved normalised rows x_norm and rstd. */
 int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const void *dout,

@@ -25,7 +25,7 @@ EXPORTS = (
     "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
     "tt_norm_profile_next_row_kernel",
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
-    "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual",
+    "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual", "tt_adaln_backward_static",
     "tt_norm_stream_probe",
 )
 
@@ -64,6 +64,7 @@ def lib() -> ctypes.CDLL:
         L.tt_adaln_backward_workspace_bytes.restype = sz
         L.tt_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
         L.tt_adaln_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
+        L.tt_adaln_backward_static.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.tt_adaln_backward_from_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_gated_residual_adaln_forward.argtypes = [vp] * 9 + [i64, i64, i64, dbl, ci, vp]
         L.tt_gated_residual_adaln_backward_workspace_bytes.restype = sz

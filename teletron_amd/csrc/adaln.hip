@@ -14,6 +14,8 @@
 // The variance is taken about the mean over the row held in registers (two
 // passes over registers, one over memory).  HBM traffic per row: forward reads
 // x and writes out (+8 B of statistics); backward reads g and x, writes dx.
+#include <atomic>
+
 #include "norm_device.h"
 #include "norm_host.h"
 
@@ -660,6 +662,61 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
                                         workspace, workspace_bytes, a)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
+}
+
+/* ---- AdaLN backward that allocates nothing: scratch in a static device array ---- */
+
+}  // extern "C"
+
+namespace ttn {
+
+// Partial column sums of tt_adaln_backward_static.  One copy per GPU the library runs on, held
+// until the process ends; every call on a GPU uses that GPU's copy.
+constexpr size_t kStaticScratchBytes = (size_t)TT_NORM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device.  The array's name is only a host-side handle;
+// its address on each GPU is looked up once, with that GPU current, and kept.
+static int static_scratch_address(void **out) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void *> cache[kMaxDevices];  // zero-initialised: null = not looked up yet
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(TT_NORM_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(TT_NORM_EINVAL, "device ordinal %d out of range", dev);
+    void *p = cache[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(TT_NORM_EHIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        cache[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return TT_NORM_OK;
+}
+
+}  // namespace ttn
+
+extern "C" {
+
+int tt_adaln_backward_static(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                             const void *scale, const float *mean, const float *rstd, int64_t batch,
+                             int64_t rows_per_sample, int64_t cols, int dtype, void *stream) {
+    int st = check_adaln_args("tt_adaln_backward_static", batch, rows_per_sample, cols, dtype, {dx, dout, x, scale});
+    if (st != TT_NORM_OK) return st;
+    const size_t need = tt_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype);
+    if (need > kStaticScratchBytes)
+        return fail(TT_NORM_EWORKSPACE,
+                    "tt_adaln_backward_static: batch=%lld rows_per_sample=%lld cols=%lld needs %zu B of scratch, the "
+                    "static array holds %zu B; use tt_adaln_backward with caller-provided scratch",
+                    (long long)batch, (long long)rows_per_sample, (long long)cols, need, kStaticScratchBytes);
+    void *ws = nullptr;
+    st = static_scratch_address(&ws);
+    if (st != TT_NORM_OK) return st;
+    // every partial row the reducer reads is written in full by the row kernel of the same call:
+    // nothing in the array has to start at zero
+    return tt_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols, dtype, ws,
+                             kStaticScratchBytes, stream);
 }
 
 /* ---- gated residual + AdaLN (3072 columns) ---- */
