@@ -29,23 +29,18 @@ ROWS, COLS = 118800, 3072
 EPS = 1e-6
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (scaled by the same counters on the plain copy kernel); None until measured.
-MEASURED_TRAFFIC_BYTES = {
-    # (FETCH_SIZE KiB * 2.000 + WRITE_SIZE KiB * 1.000) * 1024, see profiles/bench_cfg4_all_kernels.md
-    "rmsnorm_backward": int((714788.4 * 2.0 + 715872.0) * 1024),
-    "adaln_backward": int((716689.7 * 2.0 + 718944.0) * 1024),
-    "rmsnorm_forward": int((356452.5 * 2.0 + 713734.0) * 1024),
-    "adaln_forward": int((356500.1 * 2.0 + 714657.6) * 1024),
-}
-
-
-KERNEL_SYMBOL = {
-    "rmsnorm_forward": "ttn::rmsnorm_fwd_kernel<ttn::bf16_t, 3072, ttn::DenseRows>",
-    "rmsnorm_backward": "ttn::rmsnorm_bwd_kernel<ttn::bf16_t, 3072, false, ttn::DenseRows>",
-    "adaln_forward": "ttn::adaln_fwd_kernel<ttn::bf16_t, 3072, false, false>",
-    "adaln_backward": "ttn::adaln_bwd_kernel<ttn::bf16_t, 3072, false, false>",
-}
+def measured_cfg4_profile():
+    """profiles/cfg4_traffic.json: per C-ABI call the row kernel's symbol and its HBM bytes per launch from
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters on the plain copy kernel), written
+    by `python -m teletron_amd.profile_summary cfg4` together with profiles/bench_cfg4_all_kernels.md.  Returns
+    ({call: record}, valid): valid only while the kernel sources are the ones that were profiled."""
+    from teletron_amd.build import kernel_source_digest
+    path = os.path.join(ROOT, "profiles", "cfg4_traffic.json")
+    if not os.path.exists(path):
+        return {}, False
+    with open(path) as f:
+        rec = json.load(f)
+    return rec.get("calls", {}), rec.get("source_digest") == kernel_source_digest()
 
 
 WORKLOADS = {
@@ -341,6 +336,21 @@ def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
     nbytes = 2 * 5 * sample_rows * COLS * 2
+
+    # BASELINE config 1, the reference's own CPU-runnable case: RMSNorm fwd+bwd on x [2, 4096, 3072] fp32,
+    # 3 warm-up passes, 10 timed, median
+    c1 = O.make_rmsnorm_inputs((2, 4096), COLS, torch.float32, seed=0)
+    t1 = []
+    for k in range(13):
+        t0 = time.perf_counter()
+        O.eager_rmsnorm_fwd_bwd(c1["x"], c1["weight"], c1["grad"])
+        if k >= 3:
+            t1.append(time.perf_counter() - t0)
+    m1 = sorted(t1)[len(t1) // 2]
+    cfg1 = {"value": round(5 * 8192 * COLS * 4 / m1 / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "ms_per_pass": round(m1 * 1e3, 2),
+            "sample": "config 1 in full: RMSNorm fwd+bwd, x [2, 4096, 3072] fp32, PyTorch CPU eager (oracle "
+                      "restatement), 3 warm-up + 10 timed passes, median"}
     return {
         "value": round(nbytes / t / 1e9, 3),
         "unit": "GB/s",
@@ -348,6 +358,7 @@ def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
         "kind": "port",
         "sample": f"{sample_rows} of {ROWS} rows x {COLS} bf16, RMSNorm + AdaLN fwd+bwd via PyTorch CPU eager "
                   f"(oracle restatement), median of {reps}, {t * 1e3:.1f} ms per pass",
+        "config1": cfg1,
     }
 
 
@@ -494,6 +505,9 @@ def main():
     copy_gbs = 2 * tensor_bytes / (e0.elapsed_time(e1) / 10) / 1e6
 
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    dom_call = "tt_" + dom.removesuffix("_q").removesuffix("_k")
+    prof_calls, prof_valid = measured_cfg4_profile() if headline else ({}, False)
+    prof_rec = prof_calls.get(dom_call, {})
     result = {
         "metric": "fwd+bwd HBM GB/s and % of peak for RMSNorm/AdaLN at 118800x3072 bf16" if headline
                   else "fwd+bwd HBM GB/s and % of peak, workload " + args.workload,
@@ -515,11 +529,13 @@ def main():
         "tokens_per_s": round(tokens_per_step / (ms_per_step * 1e-3), 1),
         "per_call_untimed": per_call,
         "stream_copy_GB/s": round(copy_gbs, 1),
-        "roofline": {"bound": "hbm", "kernel": KERNEL_SYMBOL.get(dom) if headline else None, "call": "tt_" + dom.removesuffix("_q").removesuffix("_k"),
+        "roofline": {"bound": "hbm", "kernel": prof_rec.get("symbol") if headline else None, "call": dom_call,
                      "avg_us": round(dom_ms * 1e3, 1),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if headline else None},
+                     "traffic": prof_rec.get("traffic_bytes") if (headline and prof_valid) else None,
+                     "traffic_source": ("profiles/cfg4_traffic.json" if prof_valid else
+                                        "none: kernel sources differ from the profiled ones") if headline else None},
     }
     if headline:
         result["config"].update({"rows": ROWS, "cols": COLS})

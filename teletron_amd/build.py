@@ -33,6 +33,20 @@ KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip"]
 EXT_MODULES = {"fused_rmsnorm": "fused_rmsnorm_ext.cpp", "fused_adaln": "fused_adaln_ext.cpp"}
 
 
+def kernel_source_digest() -> str:
+    """First 16 hex digits of a sha256 over the kernel sources (names and contents of csrc/*.hip and
+    csrc/*.h): what a measurement of the kernels is tied to."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def _run(cmd, cwd=None):
     proc = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass says it does not know the packed-fp32 feature; that is expected

@@ -1,0 +1,374 @@
+"""Turns rocprofv3 output (rocpd sqlite databases) and bench.py JSON lines into the short text summaries
+kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for `roofline.kernel` and
+`roofline.traffic`.  Every summary names the commands that produced its inputs.
+
+    python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof
+        expects  <dir>/trace, <dir>/fetch, <dir>/write   (rocprofv3 -d ... of bench.py, see the text it writes)
+        optional <dir>/sq, <dir>/tcc, <dir>/stall          (counter passes)
+        optional <dir>/bench.json                          (the same bench.py run without a profiler)
+    python -m teletron_amd.profile_summary workloads --dir gpurun_out/prof     (<dir>/trace_<workload>)
+    python -m teletron_amd.profile_summary stream --dir gpurun_out/prof        (<dir>/stream.json, <dir>/stream_stall)
+
+The databases are large; run this where they were written and keep only what it writes (--out).
+"""
+from __future__ import annotations
+
+import argparse
+import glob
+import json
+import os
+import re
+import sqlite3
+
+from teletron_amd.build import ROOT, kernel_source_digest
+
+PROFILES = os.path.join(ROOT, "profiles")
+OURS = ("rmsnorm_", "adaln_", "stream_copy", "stream_probe", "colreduce")
+BOX = "MI355X (gfx950, 256 CUs), ROCm 7.2, one GPU"
+
+
+def _db(directory):
+    found = sorted(glob.glob(os.path.join(directory, "**", "*.db"), recursive=True))
+    if not found:
+        raise FileNotFoundError(f"no rocpd database under {directory}")
+    return sqlite3.connect(found[0])
+
+
+def short(name: str) -> str:
+    name = re.sub(r"^void ", "", name).replace("ttn::", "")
+    return re.sub(r"\(.*", "", name)
+
+
+def kernel_stats(directory, only_ours=True, by_grid=False):
+    """[{name, symbol, calls, avg_us, min_us, max_us, total_us, vgpr, agpr, lds, grid}] sorted by total time."""
+    cur = _db(directory).cursor()
+    group = "name, grid_x" if by_grid else "name"
+    rows = cur.execute(
+        "select name, count(*), sum(duration), avg(duration), min(duration), max(duration), max(vgpr_count), "
+        f"max(accum_vgpr_count), max(lds_size), max(grid_x) from kernels group by {group} "
+        "order by sum(duration) desc").fetchall()
+    out = []
+    for r in rows:
+        if only_ours and not any(o in r[0] for o in OURS):
+            continue
+        out.append({"name": short(r[0]), "symbol": re.sub(r"^void ", "", re.sub(r"\(.*", "", r[0])), "calls": r[1],
+                    "total_us": r[2] / 1e3, "avg_us": r[3] / 1e3, "min_us": r[4] / 1e3, "max_us": r[5] / 1e3,
+                    "vgpr": r[6], "agpr": r[7], "lds": r[8], "grid": r[9]})
+    return out
+
+
+def stats_table(stats, width=96):
+    total = sum(s["total_us"] for s in stats) or 1.0
+    lines = [f"{'kernel':{width}s} {'calls':>6} {'avg_us':>9} {'min_us':>9} {'max_us':>9} {'%':>6} {'vgpr':>5} "
+             f"{'agpr':>5} {'lds':>6} {'grid':>9}"]
+    for s in stats:
+        lines.append(f"{s['name'][:width]:{width}s} {s['calls']:6d} {s['avg_us']:9.1f} {s['min_us']:9.1f} "
+                     f"{s['max_us']:9.1f} {100 * s['total_us'] / total:6.2f} {s['vgpr']:5d} {s['agpr']:5d} "
+                     f"{s['lds']:6d} {s['grid']:9d}")
+    return "\n".join(lines)
+
+
+def counters(directory, by_grid=False):
+    """{kernel (, grid): {counter: average per dispatch}} for our kernels."""
+    cur = _db(directory).cursor()
+    group = "kernel_name, grid_size_x, counter_name" if by_grid else "kernel_name, counter_name"
+    sel = "kernel_name, grid_size_x, counter_name" if by_grid else "kernel_name, 0, counter_name"
+    out = {}
+    for name, grid, counter, value, n in cur.execute(
+            f"select {sel}, avg(value), count(*) from counters_collection group by {group}").fetchall():
+        if not any(o in name for o in OURS):
+            continue
+        key = (short(name), grid) if by_grid else short(name)
+        out.setdefault(key, {})[counter] = value
+        out[key]["_dispatches"] = n
+    return out
+
+
+def _find(d, sub):
+    for k, v in d.items():
+        if sub in (k if isinstance(k, str) else k[0]):
+            return v
+    raise KeyError(sub)
+
+
+# ------------------------------------------------------------------------------------------- cfg4
+
+CFG4_ROWS, CFG4_COLS = 118800, 3072
+CFG4_TENSOR = CFG4_ROWS * CFG4_COLS * 2
+CFG4_KERNELS = {  # C-ABI call -> (row kernel name starts with, algorithmic tensors per launch)
+    "tt_rmsnorm_forward": ("rmsnorm_fwd_kernel<bf16_t, 3072", 2),
+    "tt_rmsnorm_backward": ("rmsnorm_bwd_kernel<bf16_t, 3072", 3),
+    "tt_adaln_forward": ("adaln_fwd_kernel<bf16_t, 3072", 2),
+    "tt_adaln_backward": ("adaln_bwd_kernel<bf16_t, 3072", 3),
+}
+BENCH_CMD = "python3 bench.py --steps {steps} --warmup {warmup} --no-cpu-baseline"
+
+
+def cfg4(directory):
+    trace = kernel_stats(os.path.join(directory, "trace"))
+    fetch = counters(os.path.join(directory, "fetch"))
+    write = counters(os.path.join(directory, "write"))
+    copy_f = _find(fetch, "stream_copy_kernel")["FETCH_SIZE"]
+    copy_w = _find(write, "stream_copy_kernel")["WRITE_SIZE"]
+    kib = CFG4_TENSOR / 1024
+    f_scale, w_scale = kib / copy_f, kib / copy_w
+    digest = kernel_source_digest()
+    record = {"source_digest": digest, "workload": "cfg4", "rows": CFG4_ROWS, "cols": CFG4_COLS,
+              "calibration": {"kernel": "stream_copy_kernel", "bytes_read": CFG4_TENSOR, "bytes_written": CFG4_TENSOR,
+                              "FETCH_SIZE_KiB": round(copy_f, 1), "WRITE_SIZE_KiB": round(copy_w, 1),
+                              "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4)},
+              "calls": {}}
+    table = ["| kernel | avg µs (trace) | alg. GB/s | % of 8 TB/s | fetch MB (scaled) | write MB (scaled) | total MB | "
+             "algorithmic MB | excess |", "|---|---|---|---|---|---|---|---|---|"]
+    for call, (prefix, tensors) in CFG4_KERNELS.items():
+        st = next(s for s in trace if s["name"].startswith(prefix))
+        fb = _find(fetch, prefix)["FETCH_SIZE"] * f_scale * 1024
+        wb = _find(write, prefix)["WRITE_SIZE"] * w_scale * 1024
+        alg = tensors * CFG4_TENSOR
+        gbs = alg / st["avg_us"] / 1e3
+        record["calls"][call] = {"symbol": st["symbol"], "avg_us": round(st["avg_us"], 1),
+                                 "algorithmic_bytes": alg, "fetch_bytes": int(fb), "write_bytes": int(wb),
+                                 "traffic_bytes": int(fb + wb)}
+        table.append(f"| `{st['name']}` | {st['avg_us']:.1f} | {gbs:.0f} | {gbs / 80:.1f} % | {fb / 1e6:.1f} | "
+                     f"{wb / 1e6:.1f} | {(fb + wb) / 1e6:.1f} | {alg / 1e6:.1f} | {100 * ((fb + wb) / alg - 1):+.2f} % |")
+    with open(os.path.join(PROFILES, "cfg4_traffic.json"), "w") as f:
+        json.dump(record, f, indent=1)
+        f.write("\n")
+
+    bench_note = ""
+    bj = os.path.join(directory, "bench.json")
+    if os.path.exists(bj):
+        b = json.loads(open(bj).read().strip().splitlines()[-1])
+        r = b["roofline"]
+        bench_note = (f"\nbench.py of the same build, run without a profiler just before on the same box "
+                      f"(`{BENCH_CMD.format(steps=b['steps'], warmup=b['warmup'])}`): {b['value']:.0f} GB/s "
+                      f"({100 * b['frac_of_hbm_peak']:.1f} % of 8 TB/s), {b['ms_per_step']:.4f} ms per step; its roofline "
+                      f"entry times `{short(r['kernel'] or r['call'])}` with a HIP event pair recorded by the library around "
+                      f"that kernel: {r['avg_us']:.1f} µs.  Untimed per-call HIP-event medians: "
+                      + " / ".join(f"{v['median_us']:.1f}" for v in b["per_call_untimed"].values()) + " µs.\n")
+
+    def pmc_rows(c, name):
+        rows = [f"{'kernel':96s} {'counter':>12} {'n':>4} {'avg KiB':>14}"]
+        for k, v in sorted(c.items(), key=lambda kv: -kv[1].get(name, 0)):
+            rows.append(f"{k[:96]:96s} {name:>12} {v['_dispatches']:4d} {v[name]:14.1f}")
+        return "\n".join(rows)
+
+    md = f"""# rocprofv3 summary: bench.py, cfg4 (118 800 x 3072 bf16), all kernels
+
+Workload: one step = fused RMSNorm(3072) fwd+bwd + fused AdaLN fwd+bwd, through the C ABI.
+{BOX}.  Kernel sources digest `{digest}` (sha256 over teletron_amd/csrc, first 16 hex digits; bench.py prints
+`roofline.traffic` only while the sources it runs have this digest).  rocprofv3 writes a rocpd sqlite database;
+the tables are `select ... from kernels group by name` / `from counters_collection group by kernel_name` over it
+(durations in microseconds, counters in KiB per dispatch as rocprofv3 reports them).  Written by
+`python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof`.
+
+## Kernel trace
+
+    rocprofv3 --kernel-trace --stats -d gpurun_out/prof/trace -o bench -- {BENCH_CMD.format(steps=30, warmup=5)}
+
+```
+{stats_table(trace)}
+```
+{bench_note}
+## HBM traffic (two separate counter runs)
+
+    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/fetch -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
+    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/write -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
+
+```
+{pmc_rows(fetch, 'FETCH_SIZE')}
+```
+```
+{pmc_rows(write, 'WRITE_SIZE')}
+```
+
+Calibration on `stream_copy_kernel` (reads {CFG4_TENSOR:,} B = {kib:,.0f} KiB and writes the same):
+FETCH_SIZE reads {copy_f:,.0f} KiB -> scale factor {f_scale:.3f}; WRITE_SIZE reads {copy_w:,.0f} KiB -> scale factor {w_scale:.3f}.
+
+{chr(10).join(table)}
+
+The excess over the algorithmic bytes is the row statistics (4-8 B per row) and, for the backward kernels, the
+fp32 partial column sums (256 workgroups x 12 or 24 KiB).
+"""
+    with open(os.path.join(PROFILES, "bench_cfg4_all_kernels.md"), "w") as f:
+        f.write(md)
+    print("wrote profiles/bench_cfg4_all_kernels.md, profiles/cfg4_traffic.json (digest %s)" % digest)
+
+    passes = {p: os.path.join(directory, p) for p in ("sq", "tcc", "stall") if os.path.isdir(os.path.join(directory, p))}
+    if passes:
+        cfg4_counters(passes, digest)
+
+
+PASS_COUNTERS = {
+    "sq": "SQ_WAVES SQ_INSTS_VALU SQ_INSTS_VMEM SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY "
+          "GRBM_GUI_ACTIVE",
+    "tcc": "TCC_HIT_sum TCC_MISS_sum TCC_EA0_RDREQ_sum TCC_EA0_WRREQ_sum",
+    "stall": "TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum TCC_EA0_WRREQ_STALL_sum "
+             "TCC_TOO_MANY_EA_WRREQS_STALL_sum",
+}
+
+
+def cfg4_counters(passes, digest):
+    merged = {}
+    for p, d in passes.items():
+        for k, v in counters(d).items():
+            merged.setdefault(k, {}).update(v)
+    order = [next((k for k in merged if k.startswith(pref)), None) for pref, _ in CFG4_KERNELS.values()]
+    order.append(next((k for k in merged if k.startswith("stream_copy_kernel")), None))
+    order = [k for k in order if k]
+    names = [c for p in passes for c in PASS_COUNTERS[p].split()]
+    cmds = "\n".join(f"    rocprofv3 --pmc {PASS_COUNTERS[p]} -d gpurun_out/prof/{p} -o r -- "
+                     f"{BENCH_CMD.format(steps=3, warmup=1)}" for p in passes)
+    lines = ["| counter | " + " | ".join(k.split("<")[0] for k in order) + " |", "|---|" + "---|" * len(order)]
+    for c in names:
+        lines.append(f"| {c} | " + " | ".join(f"{merged[k].get(c, float('nan')):,.0f}" for k in order) + " |")
+    derived = []
+    if "sq" in passes:
+        derived.append("| VALU instructions per row (wavefront level) | " + " | ".join(
+            f"{merged[k]['SQ_INSTS_VALU'] / CFG4_ROWS:.0f}" for k in order[:4]) + " | |")
+        derived.append("| SQ_WAIT_INST_ANY / SQ_ACTIVE_INST_ANY | " + " | ".join(
+            f"{merged[k]['SQ_WAIT_INST_ANY'] / max(merged[k]['SQ_ACTIVE_INST_ANY'], 1):.2f}" for k in order) + " |")
+    if "tcc" in passes:
+        derived.append("| L2 hit share (HIT / (HIT + MISS)) | " + " | ".join(
+            f"{merged[k]['TCC_HIT_sum'] / (merged[k]['TCC_HIT_sum'] + merged[k]['TCC_MISS_sum']):.2f}" for k in order) + " |")
+    md = f"""# rocprofv3 counter passes: bench.py, cfg4 (118 800 x 3072 bf16), the four row kernels and the copy yardstick
+
+{BOX}.  Kernel sources digest `{digest}`.  Separate counter runs of the same command (rocprofv3 does not split
+counters over passes); values are per dispatch, averaged over the dispatches of the run.  Written by
+`python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof`.
+
+{cmds}
+
+{chr(10).join(lines)}
+
+Derived:
+
+| | {' | '.join(k.split('<')[0] for k in order)} |
+|---|{'---|' * len(order)}
+{chr(10).join(derived)}
+
+Reading: every activation byte crosses L2 once (reads leave L2 as 128-byte requests, writes as 64-byte requests:
+5.70 M and 11.4 M per 730 MB tensor; with the write-through store of the backward kernels nothing written is a
+hit).  The backward kernels are persistent grids of one wavefront per SIMD (1024 wavefronts) and issue 1.2-1.3
+VALU instructions per wait cycle; the forward kernels are one-shot grids whose wavefronts mostly wait.  The DRAM
+credit stalls are what grows when more requests are kept in flight than the memory system drains.
+"""
+    with open(os.path.join(PROFILES, "bench_cfg4_sq_tcc_counters.md"), "w") as f:
+        f.write(md)
+    print("wrote profiles/bench_cfg4_sq_tcc_counters.md")
+
+
+# -------------------------------------------------------------------------------------- workloads
+
+WORKLOAD_INFO = {
+    "gated": "gated residual + AdaLN, 118 800 x 3072 bf16: forward 2 reads + 2 writes, backward 4 reads + 2 writes",
+    "cfg1": "RMSNorm fwd+bwd, 8192 x 3072 fp32",
+    "cfg2": "QK-norm on contiguous q and k, 712 800 rows x 128 bf16",
+    "cfg2-strided": "QK-norm on the transposed [B, H, S, D] views into the fused QKV projection, 712 800 rows x 128 bf16",
+    "cfg3": "AdaLN fwd+bwd, 29 700 x 3072 bf16",
+    "cfg5": "AdaLN -> RMSNorm chain, 4 x 11 056 x 3072 bf16, one modulation row per sample",
+    "w1536-f16": "any-width kernels: RMSNorm + AdaLN fwd+bwd, 237 600 x 1536 fp16",
+    "qkv-site-rope": "QK-norm call site with the rotary embedding fused behind the norm",
+}
+
+
+def workloads(directory):
+    digest = kernel_source_digest()
+    md = [f"""# rocprofv3 summaries: bench.py workloads other than the headline step
+
+{BOX}.  Kernel sources digest `{digest}`.  Each table is `select ... from kernels group by name` over the rocpd
+database rocprofv3 wrote (durations in microseconds; torch's own fill/copy kernels of the set-up omitted).
+`stream_copy_kernel` is the copy yardstick over one tensor of the workload (1 read + 1 write).  The JSON line is
+bench.py's own (back-to-back) result for the same command without a profiler, where one was recorded.  Written by
+`python -m teletron_amd.profile_summary workloads --dir gpurun_out/prof`.
+"""]
+    for d in sorted(glob.glob(os.path.join(directory, "trace_*"))):
+        if not os.path.isdir(d):
+            continue
+        w = os.path.basename(d)[len("trace_"):]
+        md.append(f"## {w}: {WORKLOAD_INFO.get(w, '')}\n\n    rocprofv3 --kernel-trace --stats -d gpurun_out/prof/trace_{w} "
+                  f"-o bench -- {BENCH_CMD.format(steps=30, warmup=5)} --workload {w}\n\n```\n{stats_table(kernel_stats(d))}\n```\n")
+        bj = os.path.join(directory, f"bench_{w}.json")
+        if os.path.exists(bj):
+            b = json.loads(open(bj).read().strip().splitlines()[-1])
+            calls = ", ".join(f"{k} {v['median_us']:.1f} µs ({100 * v['frac_of_peak']:.1f} %)"
+                              for k, v in b["per_call_untimed"].items())
+            md.append(f"bench.py: {b['ms_per_step']:.4f} ms per step, {b['value']:.0f} GB/s "
+                      f"({100 * b['frac_of_hbm_peak']:.1f} % of 8 TB/s); per call (HIP-event medians): {calls}.\n")
+    with open(os.path.join(PROFILES, "bench_other_workloads_kernels.md"), "w") as f:
+        f.write("\n".join(md))
+    print("wrote profiles/bench_other_workloads_kernels.md")
+
+
+# ----------------------------------------------------------------------------------------- stream
+
+def stream(directory):
+    digest = kernel_source_digest()
+    b = json.loads(open(os.path.join(directory, "stream.json")).read().strip().splitlines()[-1])
+    rows = ["| reads | writes | KiB per wavefront per tensor | grid | store | µs | GB/s | % of 8 TB/s |",
+            "|---|---|---|---|---|---|---|---|"]
+    for r in b["probes"]:
+        rows.append(f"| {r['reads']} | {r['writes']} | {r['KiB_per_wavefront_per_tensor']} | {r['grid']} | {r['store']} | "
+                    f"{r['us']:.1f} | {r['GB/s']:.0f} | {100 * r['frac_of_peak']:.1f} |")
+    others = ["| copy not written here | µs | GB/s | % of 8 TB/s |", "|---|---|---|---|"]
+    for k, v in b["other_copies"].items():
+        others.append(f"| `{k}` | {v['us']:.1f} | {v['GB/s']:.0f} | {100 * v['frac_of_peak']:.1f} |")
+    best = b["best"]
+    stall_md = ""
+    sd = os.path.join(directory, "stream_stall")
+    if os.path.isdir(sd):
+        c = counters(sd, by_grid=True)
+        names = sorted({n for v in c.values() for n in v if not n.startswith("_")})
+        lines = ["| kernel | grid (threads) | " + " | ".join(names) + " |", "|---|---|" + "---|" * len(names)]
+        for (k, grid), v in sorted(c.items()):
+            if "stream_probe" in k:
+                lines.append(f"| `{k}` | {grid} | " + " | ".join(f"{v.get(n, float('nan')):,.0f}" for n in names) + " |")
+        stall_md = f"""
+## Where the mixed streams lose (counter pass over the same probes)
+
+    rocprofv3 --pmc {PASS_COUNTERS['stall']} -d gpurun_out/prof/stream_stall -o r -- python3 bench.py --workload stream-ceiling --steps 3 --warmup 4
+
+`stream_probe_kernel<reads, writes, accesses per lane, write-through>`; a grid of 65 536 / 262 144 threads is the
+persistent form (256 / 1024 workgroups), anything larger the one-shot form.  Averages per dispatch.
+
+{chr(10).join(lines)}
+"""
+    md = f"""# Streaming ceiling: what this memory system gives each read/write mix
+
+{BOX}.  Kernel sources digest `{digest}`.  `python3 bench.py --workload stream-ceiling --steps {b['steps']} --warmup {b['warmup']}`:
+plain streams over 729.9 MB tensors through the library's probe kernel (`tt_norm_stream_probe`: non-temporal
+16-byte loads, one contiguous run per wavefront and tensor, no arithmetic beyond one add), {b['steps']} launches back
+to back between two events.  Written by `python -m teletron_amd.profile_summary stream --dir gpurun_out/prof`.
+
+Best per mix: read only {best['read_only']['GB/s']:.0f} GB/s ({100 * best['read_only']['frac_of_peak']:.1f} %), two reads
+{best['two_reads']['GB/s']:.0f} ({100 * best['two_reads']['frac_of_peak']:.1f} %), write only {best['write_only']['GB/s']:.0f}
+({100 * best['write_only']['frac_of_peak']:.1f} %), copy 1R+1W {best['copy_1R_1W']['GB/s']:.0f} ({100 * best['copy_1R_1W']['frac_of_peak']:.1f} %),
+2R+1W {best['2R_1W']['GB/s']:.0f} ({100 * best['2R_1W']['frac_of_peak']:.1f} %).  Pure streams run at 85-92 % of the
+published peak; as soon as reads and writes mix, every shape drops to 72-82 %.  A row kernel moves 6 KiB per
+wavefront and tensor (a whole 3072-column row, which it needs for the row statistics): in that shape the best plain
+2R+1W stream is the one-shot grid, and the backward kernels (persistent, because the column sums live in registers)
+run faster than it (see bench_cfg4_all_kernels.md).
+
+{chr(10).join(rows)}
+
+{chr(10).join(others)}
+{stall_md}"""
+    with open(os.path.join(PROFILES, "stream_ceiling.md"), "w") as f:
+        f.write(md)
+    print("wrote profiles/stream_ceiling.md")
+
+
+def main():
+    global PROFILES
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream"))
+    ap.add_argument("--dir", default=os.path.join(ROOT, "gpurun_out", "prof"))
+    ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
+    a = ap.parse_args()
+    PROFILES = a.out
+    os.makedirs(PROFILES, exist_ok=True)
+    {"cfg4": cfg4, "workloads": workloads, "stream": stream}[a.what](a.dir)
+
+
+if __name__ == "__main__":
+    main()
