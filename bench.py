@@ -67,6 +67,14 @@ WORKLOADS = {
     "stream-ceiling": "plain streams over 729.9 MB tensors: 0-2 tensors read, 0-1 written, 1/2/6 KiB per wavefront per "
                       "tensor, one-shot and persistent grids, streaming and write-through stores; plus the runtime's "
                       "and PyTorch's copies (no normalization arithmetic: the bandwidth envelope the kernels live in)",
+    "qkv-site-rope": "the QK-norm call site including the rotary embedding the attention forward applies to q and k "
+                     "behind the norms (fp32 cos/sin tables [29700, 128]): QKVSplitNormFunction with the tables, "
+                     "forward + backward; traffic counted as 12 slice-sized tensors plus the two tables once per "
+                     "kernel launch (4 launches)",
+    "qkv-site-rope-reference": "the same call site the reference's way with these kernels: torch.split, transpose, "
+                               "contiguous copy, dense RMSNorm Function per tensor, then the rotary embedding as "
+                               "PyTorch ops (the published apply_rotary_emb formula), torch.split's backward; same "
+                               "traffic accounting as qkv-site-rope",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -190,6 +198,34 @@ def build_workload(name, torch, capi, dev):
 
         return [("eager_rmsnorm_fwd_bwd", eager_rmsnorm, 5), ("eager_adaln_fwd_bwd", eager_adaln, 5)], \
             ROWS * COLS * 2, 2 * ROWS, "bf16", grad
+    if name in ("qkv-site-rope", "qkv-site-rope-reference"):
+        from teletron_amd import fusedlayers as FL
+        B, S, H, D = 1, 29700, 24, 128
+        mixed = rnd(B, S, H, 3 * D, dtype=bf).requires_grad_(True)
+        wq = rnd(D, dtype=bf, k=0.02, bias=1.0).requires_grad_(True)
+        wk = rnd(D, dtype=bf, k=0.02, bias=1.0).requires_grad_(True)
+        gq, gk, gv = (rnd(B, H, S, D, dtype=bf) for _ in range(3))
+        ang = torch.outer(torch.arange(S, device=dev, dtype=torch.float32),
+                          1.0 / (256.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D)))
+        cos, sin = ang.cos().repeat_interleave(2, dim=1).contiguous(), ang.sin().repeat_interleave(2, dim=1).contiguous()
+
+        def fused():
+            q, k, v = FL.QKVSplitNormFunction.apply(mixed, wq, wk, EPS, cos, sin)
+            torch.autograd.backward([q, k, v], [gq, gk, gv])
+            mixed.grad = None
+
+        def reference_way():
+            q, k, v = torch.split(mixed, [D, D, D], dim=3)
+            q, k, v = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous(), v.transpose(1, 2)
+            q = FL.rotate_pairs_eager(FL.RMSNormModelFunction.apply(q, wq, EPS, D), cos, sin)
+            k = FL.rotate_pairs_eager(FL.RMSNormModelFunction.apply(k, wk, EPS, D), cos, sin)
+            torch.autograd.backward([q, k, v], [gq, gk, gv])
+            mixed.grad = None
+
+        fn = fused if name == "qkv-site-rope" else reference_way
+        slice_bytes = B * H * S * D * 2
+        tensors = 12 + 4 * (2 * S * D * 4) / slice_bytes
+        return [(name.replace("-", "_") + "_fwd_bwd", fn, tensors)], slice_bytes, S, "bf16", gq
     if name in ("qkv-site", "qkv-site-reference"):
         from teletron_amd import fusedlayers as FL
         B, S, H, D = 1, 29700, 24, 128

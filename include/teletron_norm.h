@@ -130,6 +130,31 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
                                 int64_t cols, int dtype,
                                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* The strided QK-norm with the rotary embedding the attention caller applies right behind it
+ * (teletron/models/dit/dit_attention.py:266-273 and :435-443: apply_rotary_emb(query, (freqs_cos,
+ * freqs_sin)) on the [B, H, S, D] result of q_layernorm / k_layernorm, a separate read + write pass
+ * per tensor in the reference; in the single-stream block only the first S_img tokens are rotated).
+ * x is the [n0, n1, n2, cols] view as above with n2 the token dimension; cos, sin are fp32 tables
+ * [rope_tokens, cols], row = token; tokens i2 >= rope_tokens are normalised only.  The rotation is
+ * the real-pair form of diffusers' apply_rotary_emb (use_real=True, unbind dim -1):
+ *   out[2i]   = y[2i] * cos[2i]     - y[2i+1] * sin[2i]
+ *   out[2i+1] = y[2i+1] * cos[2i+1] + y[2i]   * sin[2i+1]      (fp32, rounded once to the element type)
+ * with y the norm's output rounded to the element type.  Backward takes the gradient of the ROTATED
+ * output and returns dx and dweight of the norm.  cols must be 128 (the head dimension). */
+int tt_rmsnorm_rope_forward_strided(void *out, float *rstd, const void *x, const void *weight,
+                                    const float *cos, const float *sin, int64_t rope_tokens,
+                                    int64_t n0, int64_t n1, int64_t n2,
+                                    int64_t xs0, int64_t xs1, int64_t xs2,
+                                    int64_t cols, double eps, int dtype, void *stream);
+int tt_rmsnorm_rope_backward_strided(void *dx, void *dweight, const void *dout, const void *x,
+                                     const void *weight, const float *rstd,
+                                     const float *cos, const float *sin, int64_t rope_tokens,
+                                     int64_t n0, int64_t n1, int64_t n2,
+                                     int64_t xs0, int64_t xs1, int64_t xs2,
+                                     int64_t dxs0, int64_t dxs1, int64_t dxs2,
+                                     int64_t cols, int dtype,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+
 /* -------------------------------------------------------------------- AdaLN
  * out = round(round(LN(x) * round(1 + scale[b])) + shift[b]),  LN without affine,
  * b = row / rows_per_sample  (teletron/models/dit/dit_fusedlayers.py:198,223).

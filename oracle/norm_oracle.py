@@ -31,6 +31,11 @@ invariants of the backward (sum_c dx = 0, sum_c dx*xhat = 0), brute-force
 float64 loops on tiny inputs, torch.autograd.gradcheck, and an independent
 scalar C restatement (oracle/norm_oracle_c.c) that models the bf16 rounding
 points bit by bit.  The reference's own tests hold no vectors for this path.
+
+One function restates a third-party routine: apply_rotary_emb_real follows the
+published diffusers.models.embeddings.apply_rotary_emb (diffusers==0.32.1,
+not installed here).  It is pinned by mathematical properties only; its parity
+with the library itself is UNPINNED (see the section comment below).
 """
 from __future__ import annotations
 
@@ -99,6 +104,88 @@ def eager_gated_residual_adaln_fwd_bwd(h, attn, gate, scale, shift, grad_out, gr
     else:
         torch.autograd.backward([out, h2], [grad_out, grad_h2])
     return (h2.detach(), out.detach()) + tuple(t.grad for t in leaves)
+
+
+# --------------------------------------------------------------------------
+# rotary embedding behind the per-head norm
+# --------------------------------------------------------------------------
+# The callers (teletron/models/dit/dit_attention.py:266-273 and :435-443) rotate the normalised query and
+# key with diffusers.models.embeddings.apply_rotary_emb(x, (freqs_cos, freqs_sin)).  diffusers is a
+# third-party dependency (requirements.txt:3 pins diffusers==0.32.1) and is not installed here, so its
+# published algorithm is restated below (defaults use_real=True, use_real_unbind_dim=-1) and pinned in
+# tests/test_oracle.py by what the mathematics fixes: identity at angle 0, preservation of each pair's norm,
+# composition of angles, a brute-force complex multiplication, the inverse rotation as its gradient, and
+# negative controls for the other pairing conventions.  PARITY AGAINST THE LIBRARY ITSELF IS UNPINNED: no
+# file of the reference holds an input/output vector of this function.
+
+def apply_rotary_emb_real(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [B, H, S, D]; cos, sin [S, D] (each angle's value repeated for the two elements of its pair, as
+    get_1d_rotary_pos_embed(use_real=True) builds them, hunyuanvideo/layers.py:245-252)."""
+    cos, sin = cos[None, None], sin[None, None]
+    x_real, x_imag = x.reshape(*x.shape[:-1], -1, 2).unbind(-1)
+    x_rotated = torch.stack([-x_imag, x_real], dim=-1).flatten(3)
+    return (x.float() * cos + x_rotated.float() * sin).to(x.dtype)
+
+
+def eager_qk_norm_rope(x, weight, cos, sin, eps: float = EPS):
+    """q_layernorm / k_layernorm on the [B, H, S, D] view, then the rotary embedding on the first
+    cos.shape[0] tokens (all tokens in the double-stream block, dit_attention.py:266-273; the image tokens
+    in the single-stream block, :435-443)."""
+    y = eager_rmsnorm(x, weight, eps)
+    n = cos.shape[0]
+    if n == 0:
+        return y
+    if n == y.shape[2]:
+        return apply_rotary_emb_real(y, cos, sin)
+    return torch.cat([apply_rotary_emb_real(y[:, :, :n], cos, sin), y[:, :, n:]], dim=2)
+
+
+def eager_qk_norm_rope_fwd_bwd(x, weight, cos, sin, grad, eps: float = EPS):
+    """Returns (out, dx, dweight) as autograd produces them."""
+    xr = x.detach().clone().requires_grad_(True)
+    wr = weight.detach().clone().requires_grad_(True)
+    out = eager_qk_norm_rope(xr, wr, cos, sin, eps)
+    out.backward(grad)
+    return out.detach(), xr.grad, wr.grad
+
+
+def truth_qk_norm_rope_fwd_bwd(x, weight, cos, sin, grad, eps: float = EPS):
+    """float64, no intermediate rounding: the rotation is linear and orthogonal per pair when both elements
+    of a pair share an angle, but the general (per-element table) form is kept."""
+    n = cos.shape[0]
+    c, s = cos.double()[None, None], sin.double()[None, None]
+
+    def rot(v):
+        a, b = v[..., 0::2], v[..., 1::2]
+        out = torch.empty_like(v)
+        out[..., 0::2] = a * c[..., 0::2] - b * s[..., 0::2]
+        out[..., 1::2] = b * c[..., 1::2] + a * s[..., 1::2]
+        return out
+
+    def rot_t(g):   # transpose of rot
+        a, b = g[..., 0::2], g[..., 1::2]
+        out = torch.empty_like(g)
+        out[..., 0::2] = a * c[..., 0::2] + b * s[..., 1::2]
+        out[..., 1::2] = b * c[..., 1::2] - a * s[..., 0::2]
+        return out
+
+    y, _, _ = truth_rmsnorm_fwd_bwd(x, weight, grad, eps)
+    out = y.clone()
+    out[:, :, :n] = rot(y[:, :, :n])
+    gy = grad.double().clone()
+    gy[:, :, :n] = rot_t(gy[:, :, :n])
+    _, dx, dw = truth_rmsnorm_fwd_bwd(x, weight, gy, eps)
+    return out, dx, dw
+
+
+def make_rope_tables(tokens: int, cols: int, seed: int = 0, theta: float = 256.0):
+    """cos, sin [tokens, cols] fp32 in the layout get_1d_rotary_pos_embed(use_real=True) produces: one angle
+    per pair, repeated for both elements; angles position * theta^(-2i/cols) over a shuffled position list."""
+    g = _gen(seed + 1234)
+    pos = torch.randperm(tokens, generator=g).float()
+    inv = 1.0 / (theta ** (torch.arange(0, cols, 2).float() / cols))
+    ang = torch.outer(pos, inv)
+    return ang.cos().repeat_interleave(2, dim=1).contiguous(), ang.sin().repeat_interleave(2, dim=1).contiguous()
 
 
 # --------------------------------------------------------------------------
@@ -299,6 +386,15 @@ def adaln_excuse(x, scale, shift, want_out, eps: float = EPS) -> torch.Tensor:
     p = (xn * (1 + scale[:, None])).float().abs().reshape(want_out.shape)
     u = _ulp_rel(want_out.dtype)
     return p * (2 * u) + want_out.float().abs() * u
+
+
+def rope_excuse(y: torch.Tensor, want_out: torch.Tensor) -> torch.Tensor:
+    """Rotated norm output: a one-ulp step of either element of a pair of y moves both rotated elements by up
+    to u*(|y_even| + |y_odd|) (|cos|, |sin| <= 1), on top of the norm's own excuse and one ulp of the result."""
+    u = _ulp_rel(want_out.dtype)
+    yf = y.float().abs()
+    pair = (yf[..., 0::2] + yf[..., 1::2]).repeat_interleave(2, dim=-1)
+    return pair * (3 * u) + want_out.float().abs() * u
 
 
 def frac_outside(got: torch.Tensor, want: torch.Tensor, rtol: float, atol: float,

@@ -26,7 +26,7 @@ EXPORTS = (
     "tt_norm_profile_next_row_kernel",
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
     "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual", "tt_adaln_backward_static",
-    "tt_norm_stream_probe",
+    "tt_norm_stream_probe", "tt_rmsnorm_rope_forward_strided", "tt_rmsnorm_rope_backward_strided",
 )
 
 
@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.tt_rmsnorm_backward_from_out.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp, sz, vp]
         L.tt_rmsnorm_forward_strided.argtypes = [vp, vp, vp, vp] + [i64] * 7 + [dbl, ci, vp]
         L.tt_rmsnorm_backward_strided.argtypes = [vp] * 6 + [i64] * 10 + [ci, vp, sz, vp]
+        L.tt_rmsnorm_rope_forward_strided.argtypes = [vp] * 6 + [i64] * 8 + [dbl, ci, vp]
+        L.tt_rmsnorm_rope_backward_strided.argtypes = [vp] * 8 + [i64] * 11 + [ci, vp, sz, vp]
         L.tt_adaln_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
         L.tt_adaln_forward_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
         L.tt_adaln_backward_workspace_bytes.restype = sz
@@ -185,6 +187,40 @@ def rmsnorm_backward_strided(dout, x, weight, rstd, dx=None):
         _check(L.tt_rmsnorm_backward_strided(_p(dx), _p(dweight), _p(dout), _p(x), _p(weight), _p(rstd),
                                              n0, n1, n2, s0, s1, s2, d0, d1, d2, cols, _dt(x), _p(ws), n,
                                              _stream(x)), "tt_rmsnorm_backward_strided")
+    return dx, dweight
+
+
+def rmsnorm_rope_forward_strided(x, weight, cos, sin, eps: float):
+    """rmsnorm_forward_strided followed by the rotary embedding on tokens < cos.shape[0]; x is [..., S, D]."""
+    if not x.is_cuda or not weight.is_cuda or not weight.is_contiguous():
+        raise ValueError("tensors must live on the GPU and weight must be contiguous")
+    cols = weight.numel()
+    (n0, n1, n2), (s0, s1, s2) = _view3(x)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    rstd = torch.empty(n0 * n1 * n2, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(lib().tt_rmsnorm_rope_forward_strided(_p(out), _p(rstd), _p(x), _p(weight), _p(cos), _p(sin),
+                                                     cos.shape[0], n0, n1, n2, s0, s1, s2, cols, eps, _dt(x),
+                                                     _stream(x)), "tt_rmsnorm_rope_forward_strided")
+    return out, rstd
+
+
+def rmsnorm_rope_backward_strided(dout, x, weight, rstd, cos, sin, dx=None):
+    """dout: gradient of the rotated output (contiguous); returns (dx, dweight) of the norm."""
+    _dense_gpu(dout, weight, rstd)
+    cols = weight.numel()
+    (n0, n1, n2), (s0, s1, s2) = _view3(x)
+    dx = dense_like_layout(x) if dx is None else dx
+    _, (d0, d1, d2) = _view3(dx)
+    dweight = torch.empty_like(weight)
+    with torch.cuda.device(x.device):
+        L = lib()
+        n = L.tt_rmsnorm_backward_workspace_bytes(n0 * n1 * n2, cols, _dt(x))
+        ws = _workspace(n, x)
+        _check(L.tt_rmsnorm_rope_backward_strided(_p(dx), _p(dweight), _p(dout), _p(x), _p(weight), _p(rstd),
+                                                  _p(cos), _p(sin), cos.shape[0], n0, n1, n2, s0, s1, s2, d0, d1,
+                                                  d2, cols, _dt(x), _p(ws), n, _stream(x)),
+               "tt_rmsnorm_rope_backward_strided")
     return dx, dweight
 
 

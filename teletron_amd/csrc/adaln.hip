@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::unpack(tr[k], tv);
             E::unpack(hr[k], hv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r as x*r + (-mu*r)
+            for (int j = 0; j < VEC; ++j) v[j] = centred<T>(v[j], mu, r, nmr);
             if constexpr (WRITE_XNORM) {
                 const u32x4 xn = E::pack(v);
                 if (ok) wn.put(k * LANES, xn);
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
                     s1 += gx[j];
-                    s2 = fmaf(gx[j], FROM_XNORM ? xv[j] : fmaf(xv[j], r, nmr), s2);
+                    s2 = fmaf(gx[j], FROM_XNORM ? xv[j] : centred<T>(xv[j], mu, r, nmr), s2);
                 }
             }
         }
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
-                xn[j] = FROM_XNORM ? xv[j] : fmaf(xv[j], r, nmr);
+                xn[j] = FROM_XNORM ? xv[j] : centred<T>(xv[j], mu, r, nmr);
                 acc[1][k][j] += gv[j];
             }
             if constexpr (GATED) {

@@ -315,7 +315,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
             E::unpack(tr[k], tv);
             E::unpack(hr[k], hv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], r, nmr);  // (x - mu) * r
+            for (int j = 0; j < VEC; ++j) v[j] = centred<T>(v[j], mu, r, nmr);
             E::round(v);  // xn
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= tv[j];
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
                     s1 += gv[j];
-                    s2 = fmaf(gv[j], fmaf(xv[j], r, nmr), s2);
+                    s2 = fmaf(gv[j], centred<T>(xv[j], mu, r, nmr), s2);
                 }
             }
         }
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
-                xn[j] = fmaf(xv[j], r, nmr);
+                xn[j] = centred<T>(xv[j], mu, r, nmr);
                 acc[1][k][j] += gv[j];
             }
             if (ok && m.in[k]) wd.put(k * LANES, E::pack(o));

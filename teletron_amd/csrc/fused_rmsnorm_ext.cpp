@@ -147,7 +147,88 @@ void torch_launch_rms_backward_strided(torch::Tensor &dinp, torch::Tensor &dweig
              "tt_rmsnorm_backward_strided");
 }
 
+// ---- strided QK-norm with the rotary embedding behind it (no reference counterpart: the reference
+// runs apply_rotary_emb as separate PyTorch ops on the norm's output) ----
+static int64_t check_rope_tables(const torch::Tensor &cos, const torch::Tensor &sin, const at::Device &dev,
+                                 int64_t cols, int64_t seq) {
+    check_dense_on(cos, dev, "freqs_cos");
+    check_dense_on(sin, dev, "freqs_sin");
+    TORCH_CHECK(cos.scalar_type() == at::kFloat && sin.scalar_type() == at::kFloat, "freqs_cos/freqs_sin must be float32");
+    TORCH_CHECK(cos.dim() == 2 && cos.size(1) == cols && cos.sizes() == sin.sizes(),
+                "freqs_cos/freqs_sin must both be [tokens, ", cols, "]");
+    TORCH_CHECK(cos.size(0) <= seq, "rotary tables hold ", cos.size(0), " tokens, the view only ", seq);
+    return cos.size(0);
+}
+
+// input: a [B, H, S, D] view (or fewer leading dimensions); rows at token index >= freqs_cos.size(0) are
+// normalised but not rotated.
+void torch_launch_rms_rope_forward_strided(torch::Tensor &output, const torch::Tensor &input,
+                                           const torch::Tensor &weight, double epsilon,
+                                           torch::Tensor &inv_variance, const torch::Tensor &freqs_cos,
+                                           const torch::Tensor &freqs_sin) {
+    const auto dev = input.device();
+    TORCH_CHECK(input.is_cuda(), "input must be a GPU tensor");
+    check_dense_on(output, dev, "output");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(input, "input");
+    const int64_t cols = weight.numel();
+    const View3 v = view3(input, cols, "input");
+    const int64_t rows = v.n[0] * v.n[1] * v.n[2];
+    const int64_t tokens = check_rope_tables(freqs_cos, freqs_sin, dev, cols, v.n[2]);
+    check_elems(output, rows * cols, input.scalar_type(), "output");
+    check_elems(weight, cols, input.scalar_type(), "weight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_rmsnorm_rope_forward_strided(output.data_ptr(), inv_variance.data_ptr<float>(), input.data_ptr(),
+                                             weight.data_ptr(), freqs_cos.data_ptr<float>(),
+                                             freqs_sin.data_ptr<float>(), tokens, v.n[0], v.n[1], v.n[2], v.s[0],
+                                             v.s[1], v.s[2], cols, epsilon, dt, current_stream(input)),
+             "tt_rmsnorm_rope_forward_strided");
+}
+
+// dout: gradient of the rotated output (contiguous); dinp as in torch_launch_rms_backward_strided.
+void torch_launch_rms_rope_backward_strided(torch::Tensor &dinp, torch::Tensor &dweight, const torch::Tensor &dout,
+                                            const torch::Tensor &input, const torch::Tensor &weight,
+                                            const torch::Tensor &inv_variance, const torch::Tensor &freqs_cos,
+                                            const torch::Tensor &freqs_sin) {
+    const auto dev = dout.device();
+    TORCH_CHECK(input.is_cuda() && dinp.is_cuda(), "input and dinp must be GPU tensors");
+    TORCH_CHECK(input.device() == dev && dinp.device() == dev, "tensors are on different devices");
+    check_dense_on(dout, dev, "dout");
+    check_dense_on(dweight, dev, "dweight");
+    check_dense_on(weight, dev, "weight");
+    check_dense_on(inv_variance, dev, "inv_variance");
+    const int dt = dtype_code(dout, "dout");
+    const int64_t cols = weight.numel();
+    const View3 vx = view3(input, cols, "input");
+    const View3 vd = view3(dinp, cols, "dinp");
+    TORCH_CHECK(input.sizes() == dinp.sizes(), "dinp must have input's shape");
+    const int64_t rows = vx.n[0] * vx.n[1] * vx.n[2];
+    const int64_t tokens = check_rope_tables(freqs_cos, freqs_sin, dev, cols, vx.n[2]);
+    TORCH_CHECK(input.scalar_type() == dout.scalar_type() && dinp.scalar_type() == dout.scalar_type(),
+                "input, dinp and dout must share a dtype");
+    check_elems(dout, rows * cols, dout.scalar_type(), "dout");
+    check_elems(weight, cols, dout.scalar_type(), "weight");
+    check_elems(dweight, cols, dout.scalar_type(), "dweight");
+    check_elems(inv_variance, rows, at::kFloat, "inv_variance");
+    c10::DeviceGuard guard(dev);
+    const size_t need = tt_rmsnorm_backward_workspace_bytes(rows, cols, dt);
+    TORCH_CHECK(need > 0 || rows == 0, "unsupported RMSNorm shape: cols=", cols);
+    at::Tensor ws = scratch(need, dout);
+    raise_on(tt_rmsnorm_rope_backward_strided(dinp.data_ptr(), dweight.data_ptr(), dout.data_ptr(), input.data_ptr(),
+                                              weight.data_ptr(), inv_variance.data_ptr<float>(),
+                                              freqs_cos.data_ptr<float>(), freqs_sin.data_ptr<float>(), tokens,
+                                              vx.n[0], vx.n[1], vx.n[2], vx.s[0], vx.s[1], vx.s[2], vd.s[0], vd.s[1],
+                                              vd.s[2], cols, dt, ws.data_ptr(), need, current_stream(dout)),
+             "tt_rmsnorm_rope_backward_strided");
+}
+
 PYBIND11_MODULE(fused_rmsnorm, m) {
+    m.def("torch_launch_rms_rope_forward_strided", &torch_launch_rms_rope_forward_strided,
+          "strided RMSNorm forward with the rotary embedding applied to the result");
+    m.def("torch_launch_rms_rope_backward_strided", &torch_launch_rms_rope_backward_strided,
+          "backward of the strided RMSNorm + rotary embedding");
     m.def("torch_launch_rms_forward", &torch_launch_rms_forward, "RMSNorm forward kernel");
     m.def("torch_launch_rms_backward", &torch_launch_rms_backward,
           "RMSNorm backward kernel (from the saved forward output)");

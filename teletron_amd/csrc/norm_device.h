@@ -214,6 +214,18 @@ __device__ __forceinline__ void wait_memory_ops() {
 }
 
 
+// xhat = (x - mu) * r.  Two-byte element types take it as one fused multiply-add, x*r + (-mu*r): the
+// rounding of mu*r (half an fp32 ulp of |mu|*r) is far below what the result is rounded to next.
+// Four-byte rows subtract first, as the eager LayerNorm does: for a row whose mean is many standard
+// deviations away, the fused form would cost a few fp32 ulps of |mu|*r in every element.
+template <typename T>
+__device__ __forceinline__ float centred(float x, float mu, float r, float nmr) {
+    if constexpr (sizeof(T) == 4)
+        return (x - mu) * r;
+    else
+        return fmaf(x, r, nmr);
+}
+
 // Makes the compiler forget what it knows about a packed register array (no
 // instruction is emitted).  Used on loop-invariant packed parameters at the
 // top of each row iteration: without it the unpacked fp32 copies are hoisted

@@ -58,6 +58,7 @@ struct RowAddr {
     int64_t row;   // logical row number
     int64_t xoff;  // element offset of the row in x
     int64_t doff;  // element offset of the row in dx (backward only)
+    int64_t seq;   // index along the view's last leading dimension (the token of a [B, H, S, D] view)
     bool ok;
 };
 
@@ -72,6 +73,7 @@ struct DenseRows {
         a.row = grp * RPW + sub;
         a.ok = a.row < rows;
         a.xoff = a.doff = a.row * C;
+        a.seq = a.row;
         return a;
     }
 };
@@ -99,6 +101,7 @@ struct Strided3Rows {
         const int64_t i0 = q / tiles2;
         RowAddr a;
         a.ok = i2 < n2;
+        a.seq = i2;
         a.row = (i0 * n1 + i1) * n2 + i2;
         a.xoff = i0 * xs0 + i1 * xs1 + i2 * xs2;
         a.doff = i0 * ds0 + i1 * ds1 + i2 * ds2;
@@ -106,10 +109,68 @@ struct Strided3Rows {
     }
 };
 
-template <typename T, int C, typename Map>
+// ---- rotary embedding behind the norm -----------------------------------------
+// The attention caller rotates the normalised query and key right after the per-head norm
+// (teletron/models/dit/dit_attention.py:266-273, :435-443) with the real-pair form of
+// diffusers' apply_rotary_emb: for tokens below `tokens`
+//     out = cast(float(y) * cos + float(rotate_pairs(y)) * sin),   rotate_pairs(y)[2i, 2i+1] = (-y[2i+1], y[2i])
+// with cos, sin fp32 tables [tokens, C]; each product and the sum are rounded to fp32, the result
+// once to the element type.  Pairs are adjacent, so both halves sit in one lane's 16-byte piece.
+struct NoRope {
+    static constexpr bool kOn = false;
+};
+struct RopeTable {
+    static constexpr bool kOn = true;
+    const float *cos, *sin;  // [tokens, C] fp32, row = token index
+    int64_t tokens;          // rows of the view at sequence index >= tokens are left unrotated
+};
+
+template <int VEC>
+__device__ __forceinline__ void load_fp32_run(float (&dst)[VEC], const float *p) {
+#pragma unroll
+    for (int i = 0; i < VEC / 4; ++i) {
+        const u32x4 t = load16(reinterpret_cast<const u32x4 *>(p) + i);  // cached: every head reuses the row
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[4 * i + j] = as_f32(t[j]);
+    }
+}
+
+// y -> y*cos + rotate_pairs(y)*sin in fp32 (y already rounded to the element type)
+template <int VEC>
+__device__ __forceinline__ void rotate_pairs_forward(float (&v)[VEC], const float (&c)[VEC], const float (&s)[VEC]) {
+#pragma unroll
+    for (int j = 0; j < VEC; j += 2) {
+        const float a = v[j], b = v[j + 1];
+        v[j] = a * c[j] - b * s[j];
+        v[j + 1] = b * c[j + 1] + a * s[j + 1];
+    }
+}
+
+// The gradient of the rotation as autograd forms it: g*cos and g*sin are each cast to the element
+// type (the two branches of x.float() and rotate_pairs(x).float()), the latter routed back through
+// the pair swap, and the two contributions are added in the element type.
+template <typename E, int VEC>
+__device__ __forceinline__ void rotate_pairs_backward(float (&g)[VEC], const float (&c)[VEC], const float (&s)[VEC]) {
+    float direct[VEC], swapped[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        direct[j] = g[j] * c[j];
+        swapped[j] = g[j] * s[j];
+    }
+    E::round(direct);
+    E::round(swapped);
+#pragma unroll
+    for (int j = 0; j < VEC; j += 2) {
+        g[j] = direct[j] + swapped[j + 1];
+        g[j + 1] = direct[j + 1] - swapped[j];
+    }
+    E::round(g);
+}
+
+template <typename T, int C, typename Map, typename Rope = NoRope>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 ? 4 : 3) void rmsnorm_fwd_kernel(
     T *__restrict__ out, float *__restrict__ rstd, const T *__restrict__ x,
-    const T *__restrict__ w, const Map map, float eps) {
+    const T *__restrict__ w, const Map map, float eps, const Rope rope = Rope{}) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
@@ -159,6 +220,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             E::round(v);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+            if constexpr (Rope::kOn) {
+                if (ok && at.seq < rope.tokens) {
+                    float cv[VEC], sv[VEC];
+                    const int64_t col0 = at.seq * C + (k * LANES + l) * VEC;
+                    load_fp32_run<VEC>(cv, rope.cos + col0);
+                    load_fp32_run<VEC>(sv, rope.sin + col0);
+                    E::round(v);  // the norm's output in the element type, which the rotation reads
+                    rotate_pairs_forward<VEC>(v, cv, sv);
+                }
+            }
             if (ok) wo.put(k * LANES, E::pack(v));
         }
     }
@@ -173,11 +244,13 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 // processed (two row buffers, ping-pong).  Few, fat, always-loading wavefronts
 // keep about 48 KiB of reads in flight per compute unit, which is where this
 // memory system streams best; more resident wavefronts only add queueing.
-template <typename T, int C, bool FROM_OUT, typename Map>
+// Rope::kOn: dout is the gradient of the ROTATED output; it is turned back through the rotation
+// (rotate_pairs_backward) as the row arrives, and everything below sees the gradient of the norm's output.
+template <typename T, int C, bool FROM_OUT, typename Map, typename Rope = NoRope>
 __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN_BWD_WAVES_PER_SIMD : 4) void rmsnorm_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g,
     const T *__restrict__ xin, const T *__restrict__ w, const float *__restrict__ rstd,
-    const Map map) {
+    const Map map, const Rope rope = Rope{}) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
@@ -217,11 +290,13 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         float r;
         int64_t doff0;   // element offset in dx of the wavefront's first row (wave-uniform)
         uint32_t dlane;  // this lane's byte offset from there
+        int64_t seq;     // token index (rotary form only)
         bool ok;
     };
     auto fetch = [&](RowRegs &b, int64_t grp) {
         const RowAddr at = map.template locate<RPW, C>(grp, sub);
         b.ok = at.ok;
+        b.seq = at.seq;
         b.doff0 = map.template locate<RPW, C>(grp, 0).doff;
         b.dlane = (uint32_t)((at.doff - b.doff0) * (int64_t)sizeof(T)) + l * 16;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
@@ -240,8 +315,23 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
 #endif
         b.r = b.ok ? rstd[at.row] : 0.0f;
     };
-    auto process = [&](const RowRegs &b, auto &&between_passes) {
+    auto process = [&](RowRegs &b, auto &&between_passes) {
         const float r = b.r;
+        if constexpr (Rope::kOn) {
+            // dout arrives as the gradient of the rotated output: back through the rotation first
+            if (b.ok && b.seq < rope.tokens) {
+#pragma unroll
+                for (int k = 0; k < CHUNKS; ++k) {
+                    float gv[VEC], cv[VEC], sv[VEC];
+                    const int64_t col0 = b.seq * C + (k * LANES + l) * VEC;
+                    load_fp32_run<VEC>(cv, rope.cos + col0);
+                    load_fp32_run<VEC>(sv, rope.sin + col0);
+                    E::unpack(b.g[k], gv);
+                    rotate_pairs_backward<E, VEC>(gv, cv, sv);
+                    b.g[k] = E::pack(gv);
+                }
+            }
+        }
         // pass 1: gy = rnd(g*w), kept packed in the element type; row dot  sum_c gy * xs
         //   xs = x (native) or xhat = out / w (from the saved output)
         u32x4 gyp[CHUNKS];
@@ -319,9 +409,9 @@ struct RmsTune {
     static constexpr int kBwdBlocksPerCu = TTN_RMS_BWD_BLOCKS_PER_CU;
 };
 
-template <typename T, int C, typename Map>
+template <typename T, int C, typename Map, typename Rope = NoRope>
 static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *w, const Map &map,
-                             int64_t rows, double eps, hipStream_t stream) {
+                             int64_t rows, double eps, hipStream_t stream, const Rope &rope = Rope{}) {
     if (rows == 0) return TT_NORM_OK;  // empty input: nothing to do
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
@@ -330,8 +420,8 @@ static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "rmsnorm forward: grid too large");
     {
         RowKernelProfile prof(stream);
-        rmsnorm_fwd_kernel<T, C, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_RMS_FWD_DYN_LDS, stream>>>(
-            (T *)out, rstd, (const T *)x, (const T *)w, map, (float)eps);
+        rmsnorm_fwd_kernel<T, C, Map, Rope><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_RMS_FWD_DYN_LDS, stream>>>(
+            (T *)out, rstd, (const T *)x, (const T *)w, map, (float)eps, rope);
     }
     return check_launch("rmsnorm forward launch");
 }
@@ -343,10 +433,10 @@ static RowPlan rmsnorm_backward_plan(int64_t rows, int cus) {
     return make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kBwdBlocksPerCu, cus);
 }
 
-template <typename T, int C, bool FROM_OUT, typename Map>
+template <typename T, int C, bool FROM_OUT, typename Map, typename Rope = NoRope>
 static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin, const void *w,
                               const float *rstd, const Map &map, int64_t rows, int dtype, void *ws,
-                              size_t ws_bytes, hipStream_t stream) {
+                              size_t ws_bytes, hipStream_t stream, const Rope &rope = Rope{}) {
     // empty input: dweight is the empty sum, written by the reducer over zero partial rows
     if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, nullptr, 1, 0, C, C, dtype, stream);
     int st = TT_NORM_OK;
@@ -358,8 +448,8 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
     {
         RowKernelProfile prof(stream);
-        rmsnorm_bwd_kernel<T, C, FROM_OUT, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-            (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, map);
+        rmsnorm_bwd_kernel<T, C, FROM_OUT, Map, Rope><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+            (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)w, rstd, map, rope);
     }
     st = check_launch("rmsnorm backward launch");
     if (st != TT_NORM_OK) return st;
@@ -510,6 +600,68 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
                                            workspace_bytes, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
+}
+
+/* ---- strided QK-norm with the rotary embedding applied behind it (head dimension 128) ---- */
+
+static int check_rope(const char *who, int64_t cols, const float *cos, const float *sin, int64_t rope_tokens,
+                      int64_t n2) {
+    if (cols != 128) return fail(TT_NORM_EUNSUPPORTED, "%s: built for cols 128 (the head dimension) only", who);
+    if (rope_tokens < 0 || rope_tokens > n2)
+        return fail(TT_NORM_EINVAL, "%s: rope_tokens=%lld outside [0, n2=%lld]", who, (long long)rope_tokens, (long long)n2);
+    if (rope_tokens > 0 && (!cos || !sin)) return fail(TT_NORM_EINVAL, "%s: null cos/sin table", who);
+    if (!aligned16(cos) || !aligned16(sin)) return fail(TT_NORM_EALIGN, "%s: cos/sin table not 16-byte aligned", who);
+    return TT_NORM_OK;
+}
+
+int tt_rmsnorm_rope_forward_strided(void *out, float *rstd, const void *x, const void *weight, const float *cos,
+                                    const float *sin, int64_t rope_tokens, int64_t n0, int64_t n1, int64_t n2,
+                                    int64_t xs0, int64_t xs1, int64_t xs2, int64_t cols, double eps, int dtype,
+                                    void *stream) {
+    const int64_t xs[3] = {xs0, xs1, xs2};
+    int st = check_strided("tt_rmsnorm_rope_forward_strided", n0, n1, n2, cols, dtype, xs, "x");
+    if (st != TT_NORM_OK) return st;
+    const int64_t rows = n0 * n1 * n2;
+    st = check_rms_args("tt_rmsnorm_rope_forward_strided", rows, cols, dtype, {out, x, weight}, true);
+    if (st == TT_NORM_OK) st = check_rope("tt_rmsnorm_rope_forward_strided", cols, cos, sin, rope_tokens, n2);
+    if (st != TT_NORM_OK) return st;
+    if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_rope_forward_strided: null rstd");
+    const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, 0, 0, 0};
+    const RopeTable rope{cos, sin, rope_tokens};
+    const hipStream_t s = (hipStream_t)stream;
+    if (dtype == TT_NORM_BF16)
+        return rmsnorm_forward_t<bf16_t, 128, Strided3Rows, RopeTable>(out, rstd, x, weight, map, rows, eps, s, rope);
+    if (dtype == TT_NORM_F16)
+        return rmsnorm_forward_t<f16_t, 128, Strided3Rows, RopeTable>(out, rstd, x, weight, map, rows, eps, s, rope);
+    return rmsnorm_forward_t<float, 128, Strided3Rows, RopeTable>(out, rstd, x, weight, map, rows, eps, s, rope);
+}
+
+int tt_rmsnorm_rope_backward_strided(void *dx, void *dweight, const void *dout, const void *x, const void *weight,
+                                     const float *rstd, const float *cos, const float *sin, int64_t rope_tokens,
+                                     int64_t n0, int64_t n1, int64_t n2, int64_t xs0, int64_t xs1, int64_t xs2,
+                                     int64_t dxs0, int64_t dxs1, int64_t dxs2, int64_t cols, int dtype,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+    const int64_t xs[3] = {xs0, xs1, xs2}, ds[3] = {dxs0, dxs1, dxs2};
+    int st = check_strided("tt_rmsnorm_rope_backward_strided", n0, n1, n2, cols, dtype, xs, "x");
+    if (st == TT_NORM_OK) st = check_strided("tt_rmsnorm_rope_backward_strided", n0, n1, n2, cols, dtype, ds, "dx");
+    if (st != TT_NORM_OK) return st;
+    const int64_t rows = n0 * n1 * n2;
+    st = check_rms_args("tt_rmsnorm_rope_backward_strided", rows, cols, dtype, {dx, dout, x, weight}, true);
+    if (st == TT_NORM_OK) st = check_rope("tt_rmsnorm_rope_backward_strided", cols, cos, sin, rope_tokens, n2);
+    if (st != TT_NORM_OK) return st;
+    if (!dweight || (!rstd && rows > 0))
+        return fail(TT_NORM_EINVAL, "tt_rmsnorm_rope_backward_strided: null dweight/rstd");
+    const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, dxs0, dxs1, dxs2};
+    const RopeTable rope{cos, sin, rope_tokens};
+    const hipStream_t s = (hipStream_t)stream;
+    if (dtype == TT_NORM_BF16)
+        return rmsnorm_backward_t<bf16_t, 128, false, Strided3Rows, RopeTable>(dx, dweight, dout, x, weight, rstd, map, rows,
+                                                                               dtype, workspace, workspace_bytes, s, rope);
+    if (dtype == TT_NORM_F16)
+        return rmsnorm_backward_t<f16_t, 128, false, Strided3Rows, RopeTable>(dx, dweight, dout, x, weight, rstd, map, rows,
+                                                                              dtype, workspace, workspace_bytes, s, rope);
+    return rmsnorm_backward_t<float, 128, false, Strided3Rows, RopeTable>(dx, dweight, dout, x, weight, rstd, map, rows, dtype,
+                                                                          workspace, workspace_bytes, s, rope);
 }
 
 }  // extern "C"

@@ -342,7 +342,10 @@ class _AdaLNZeroBase(nn.Module):
             if not cols_supported(embedding_dim, torch.float32):  # the strictest element size
                 raise ValueError(f"fused_kernels=True: {_unsupported(embedding_dim, torch.float32)}")
             _require_extension(fused_adaln, "fused_adaln")
-            self.adaLN = AdaLNCustom(embedding_dim, eps=1e-6)
+            # the fused kernel stands in for the eager norm the constructor would otherwise build, with that
+            # norm's eps: 1e-6 for nn.LayerNorm as built below, nn.LayerNorm's default 1e-5 for FP32LayerNorm
+            # (the reference's fused branch always passes 1e-6, dit_fusedlayers.py:194-195)
+            self.adaLN = AdaLNCustom(embedding_dim, eps=1e-5 if norm_type == "fp32_layer_norm" else 1e-6)
         elif norm_type == "layer_norm":
             self.norm = nn.LayerNorm(embedding_dim, elementwise_affine=False, eps=1e-6)
         elif norm_type == "fp32_layer_norm":
@@ -503,8 +506,15 @@ class QKVSplitNormFunction(Function):
     D must be 128 or 3072."""
 
     @staticmethod
-    def forward(ctx, mixed_qkv, weight_q, weight_k, epsilon):
+    def forward(ctx, mixed_qkv, weight_q, weight_k, epsilon, *rotary):
+        """rotary: nothing, or (freqs_cos, freqs_sin) as the attention forward receives them
+        (dit_attention.py:244-245): float32 [S_img, D].  q and k are then also rotated the way
+        apply_rotary_emb does behind q_layernorm / k_layernorm (dit_attention.py:266-273), for the first
+        S_img tokens (all of them in the double-stream block, the image part in the single-stream block,
+        :435-443), inside the same kernels."""
         ext = _require_extension(fused_rmsnorm, "fused_rmsnorm")
+        if len(rotary) not in (0, 2):
+            raise ValueError("pass freqs_cos and freqs_sin together, or neither")
         _require_gpu(mixed_qkv, "QKVSplitNormFunction")
         if mixed_qkv.dim() != 4 or mixed_qkv.shape[-1] % 3:
             raise ValueError(f"mixed_qkv must be [B, S, H, 3*D], got {tuple(mixed_qkv.shape)}")
@@ -512,6 +522,15 @@ class QKVSplitNormFunction(Function):
         if cols not in TUNED_COLS or mixed_qkv.dtype not in _ELEM_BYTES:
             raise ValueError(f"QKVSplitNormFunction needs D in {TUNED_COLS} and bfloat16/float16/float32, got D={cols}, "
                              f"{mixed_qkv.dtype}")
+        tables = None
+        if rotary:
+            if cols != 128:
+                raise ValueError(f"the fused rotary embedding is built for head dimension 128, got {cols}")
+            tables = tuple(_aligned_contiguous(t.to(device=mixed_qkv.device, dtype=torch.float32)) for t in rotary)
+            if tables[0].dim() != 2 or tables[0].shape != tables[1].shape or tables[0].shape[1] != cols \
+                    or tables[0].shape[0] > mixed_qkv.shape[1]:
+                raise ValueError(f"freqs_cos/freqs_sin must both be [S_img <= {mixed_qkv.shape[1]}, {cols}], got "
+                                 f"{tuple(tables[0].shape)} and {tuple(tables[1].shape)}")
         if weight_q.numel() != cols or weight_k.numel() != cols:
             raise ValueError(f"weights must have {cols} elements")
         mixed = mixed_qkv if mixed_qkv.is_contiguous() and mixed_qkv.data_ptr() % 16 == 0 else \
@@ -523,11 +542,15 @@ class QKVSplitNormFunction(Function):
         for x, w in ((q_in, ws[0]), (k_in, ws[1])):
             out = torch.empty((B, H, S, cols), dtype=mixed.dtype, device=mixed.device)
             invvar = torch.empty(B * H * S, device=mixed.device, dtype=torch.float32)
-            ext.torch_launch_rms_forward_strided(out, x, w, float(epsilon), invvar)
+            if tables is None:
+                ext.torch_launch_rms_forward_strided(out, x, w, float(epsilon), invvar)
+            else:
+                ext.torch_launch_rms_rope_forward_strided(out, x, w, float(epsilon), invvar, tables[0], tables[1])
             outs.append(out)
             stats.append(invvar)
-        ctx.save_for_backward(mixed, ws[0], ws[1], stats[0], stats[1])
+        ctx.save_for_backward(mixed, ws[0], ws[1], stats[0], stats[1], *(tables or ()))
         ctx.cols = cols
+        ctx.n_rotary = len(rotary)
         ctx.w_meta = [(w.shape, w.dtype) for w in (weight_q, weight_k)]
         ctx.set_materialize_grads(False)
         # v leaves as a copy-free view only when mixed_qkv itself was usable in place
@@ -536,7 +559,7 @@ class QKVSplitNormFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_q, grad_k, grad_v):
-        mixed, wq, wk, rstd_q, rstd_k = ctx.saved_tensors
+        mixed, wq, wk, rstd_q, rstd_k, *tables = ctx.saved_tensors
         cols = ctx.cols
         d_mixed = torch.empty_like(mixed)
         slices = [d_mixed[..., i * cols:(i + 1) * cols].transpose(1, 2) for i in range(3)]
@@ -549,27 +572,49 @@ class QKVSplitNormFunction(Function):
             else:
                 g = _aligned_contiguous(g.to(mixed.dtype))
                 x = mixed[..., i * cols:(i + 1) * cols].transpose(1, 2)
-                fused_rmsnorm.torch_launch_rms_backward_strided(slices[i], dw, g, x, w, rstd)
+                if tables:
+                    fused_rmsnorm.torch_launch_rms_rope_backward_strided(slices[i], dw, g, x, w, rstd, *tables)
+                else:
+                    fused_rmsnorm.torch_launch_rms_backward_strided(slices[i], dw, g, x, w, rstd)
             shape, dtype = ctx.w_meta[i]
             grads_w.append(dw.reshape(shape).to(dtype))
         if grad_v is None:
             slices[2].zero_()
         else:
             slices[2].copy_(grad_v)
-        return d_mixed, grads_w[0], grads_w[1], None
+        return (d_mixed, grads_w[0], grads_w[1], None) + (None,) * ctx.n_rotary
 
 
-def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSNorm"):
+def rotate_pairs_eager(x: torch.Tensor, freqs_cos: torch.Tensor, freqs_sin: torch.Tensor) -> torch.Tensor:
+    """What the reference's callers get from diffusers' apply_rotary_emb(x, (freqs_cos, freqs_sin)) with its
+    defaults (real tables, pairs unbound along the last dimension): x [B, H, S, D], tables [S, D]."""
+    cos, sin = freqs_cos[None, None].to(x.device), freqs_sin[None, None].to(x.device)
+    x_real, x_imag = x.reshape(*x.shape[:-1], -1, 2).unbind(-1)
+    x_rotated = torch.stack([-x_imag, x_real], dim=-1).flatten(3)
+    return (x.float() * cos + x_rotated.float() * sin).to(x.dtype)
+
+
+def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSNorm", rotary=None):
     """query, key, value as `[B, H, S, D]` from the fused projection `[B, S, H, 3*D]`: the split, the
-    transposes and the two per-head RMSNorms of dit_attention.py:149-214 in one call.  Fused when
-    FUSED_KERNELS is on and the head dimension is one the tuned kernels take; the reference's own
-    sequence of operations otherwise."""
+    transposes and the two per-head RMSNorms of dit_attention.py:149-214 in one call, and with
+    rotary=(freqs_cos, freqs_sin) also the rotary embedding of query and key that follows them
+    (dit_attention.py:266-273; tables of S_img <= S rows rotate the first S_img tokens, :435-443).
+    Fused when FUSED_KERNELS is on and the head dimension is one the tuned kernels take (128 for the
+    rotary form); the reference's own sequence of operations otherwise."""
     D = mixed_qkv.shape[-1] // 3
-    if (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in _ELEM_BYTES
-            and q_norm.eps == k_norm.eps):
+    fusable = (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in _ELEM_BYTES
+               and q_norm.eps == k_norm.eps)
+    if fusable and rotary is None:
         return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
+    if fusable and D == 128:
+        return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps, *rotary)
     query, key, value = torch.split(mixed_qkv, [D, D, D], dim=3)
-    return q_norm(query.transpose(1, 2)), k_norm(key.transpose(1, 2)), value.transpose(1, 2)
+    query, key, value = q_norm(query.transpose(1, 2)), k_norm(key.transpose(1, 2)), value.transpose(1, 2)
+    if rotary is not None:
+        n = rotary[0].shape[0]
+        query = torch.cat([rotate_pairs_eager(query[:, :, :n], *rotary), query[:, :, n:]], dim=2)
+        key = torch.cat([rotate_pairs_eager(key[:, :, :n], *rotary), key[:, :, n:]], dim=2)
+    return query, key, value
 
 
 def Get_RMSNorm():

@@ -159,8 +159,14 @@ def test_modulated_layer_norm_matches_unfused_norm2_site(FL, gpu_device):
     d = O.make_adaln_inputs(2, 200, 3072, torch.bfloat16, seed=46)
     ln = torch.nn.LayerNorm(3072, elementwise_affine=False, eps=1e-6)
     want = ln(d["x"]) * (1 + d["scale"][:, None]) + d["shift"][:, None]
-    got = FL.modulated_layer_norm(d["x"].to(gpu_device), d["scale"].to(gpu_device), d["shift"].to(gpu_device))
+    xg, sg, hg = (d[k].to(gpu_device).requires_grad_(True) for k in ("x", "scale", "shift"))
+    got = FL.modulated_layer_norm(xg, sg, hg)
     fwd_ok(got, want, O.adaln_excuse(d["x"], d["scale"], d["shift"], want))
+    got.backward(d["grad"].to(gpu_device))
+    _, want_dx, want_ds, want_dh = O.eager_adaln_fwd_bwd(d["x"], d["scale"], d["shift"], d["grad"])
+    grad_ok(xg.grad, want_dx, allow=1e-5)
+    grad_ok(sg.grad, want_ds)
+    grad_ok(hg.grad, want_dh)
 
 
 def test_adaln_keeping_the_residual_stream(FL, gpu_device):
@@ -248,10 +254,21 @@ def test_adaln_continuous_fused_vs_eager_branch(FL, gpu_device):
         torch.testing.assert_close(want, ref)
         mod = FL.modulated_layer_norm(x.to(gpu_device).transpose(0, 1), scale.to(gpu_device), shift.to(gpu_device))
         fwd_ok(mod.transpose(0, 1), ref, O.adaln_excuse(x.transpose(0, 1), scale, shift, ref.transpose(0, 1)).transpose(0, 1))
-        assert (got.detach().cpu().float() - want.float()).abs().max() <= 0.1 * want.float().abs().max()
-        got.backward(torch.ones_like(got))
-        assert xg.grad.shape == x.shape and torch.isfinite(xg.grad.float()).all()
-        assert fused.adaLN_modulation[1].weight.grad is not None
+        # the module itself, forward and backward, on the modulation rows ITS OWN linear produced on the GPU
+        rows_g = fused.adaLN_modulation(cond.to(gpu_device)).detach().cpu()
+        sc_g, sh_g = rows_g[:, :C].contiguous(), rows_g[:, C:].contiguous()
+        g = torch.randn(S, B, C, generator=torch.Generator().manual_seed(77 + B)).bfloat16()
+        w_out, w_dx, w_ds, w_dh = O.eager_adaln_fwd_bwd(x.transpose(0, 1).contiguous(), sc_g, sh_g,
+                                                        g.transpose(0, 1).contiguous(), 1e-6)
+        fwd_ok(got.transpose(0, 1), w_out, O.adaln_excuse(x.transpose(0, 1).contiguous(), sc_g, sh_g, w_out))
+        got.backward(g.to(gpu_device))
+        assert xg.grad.shape == x.shape
+        grad_ok(xg.grad.transpose(0, 1).contiguous(), w_dx, allow=1e-5)
+        # dscale/dshift reach the modulation linear: its weight gradient is [dscale, dshift]^T @ silu(cond)
+        act = torch.nn.functional.silu(cond.float())
+        want_w = torch.cat([w_ds.float(), w_dh.float()], dim=1).t() @ act
+        got_w = fused.adaLN_modulation[1].weight.grad.float().cpu()
+        assert (got_w - want_w).abs().max() <= 2e-2 * want_w.abs().max()
 
 
 def test_reference_signature_extension_calls(FL, gpu_device):
@@ -464,3 +481,154 @@ def test_block_norm_path_composed_from_the_fused_functions(FL, gpu_device):
         got = gpu[name].grad.cpu()
         scale = want.abs().max()
         assert (got - want).abs().max() <= 2e-4 * scale + 1e-5, (name, float((got - want).abs().max()), float(scale))
+
+
+# -------------------------------------------------- the FP32LayerNorm variant
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("C", [3072, 1536])
+def test_fp32_layer_norm_variant_is_the_same_kernel_at_eps_1e5(FL, gpu_device, dtype, C):
+    """norm_type="fp32_layer_norm" (dit_fusedlayers.py:48-57,200-201,253-254): LayerNorm evaluated in fp32 and
+    cast back, built without eps (so 1e-5), then modulated in the input dtype.  The fused kernel always
+    normalises in fp32 and rounds once, so it is this variant when called with eps 1e-5: forward and
+    backward against autograd through FP32LayerNorm on the CPU."""
+    B, S = 2, 257
+    d = O.make_adaln_inputs(B, S, C, dtype, seed=81)
+    d["x"] = (d["x"].float() * 0.02).to(dtype)          # small rows: var ~ 4e-4, where eps 1e-5 vs 1e-6 is visible
+    ln = FL.FP32LayerNorm(C, elementwise_affine=False, bias=False)
+    assert ln.eps == 1e-5
+    leaves = [d[k].clone().requires_grad_(True) for k in ("x", "scale", "shift")]
+    want = ln(leaves[0]) * (1 + leaves[1][:, None]) + leaves[2][:, None]
+    want.backward(d["grad"])
+    xg, sg, hg = (d[k].to(gpu_device).requires_grad_(True) for k in ("x", "scale", "shift"))
+    got = FL.modulated_layer_norm(xg, sg, hg, eps=1e-5)
+    got.backward(d["grad"].to(gpu_device))
+    fwd_ok(got, want.detach(), O.adaln_excuse(d["x"], d["scale"], d["shift"], want.detach(), 1e-5))
+    terms = O.adaln_dx_terms(d["x"], d["scale"], d["grad"], 1e-5)
+    assert O.frac_outside(xg.grad.cpu(), leaves[0].grad, 1e-2, 1e-3, magnitude=terms) <= 1e-5
+    grad_ok(sg.grad, leaves[1].grad)
+    grad_ok(hg.grad, leaves[2].grad)
+    # and eps matters at this row size: the eps 1e-6 kernel is visibly something else
+    other = FL.modulated_layer_norm(xg.detach(), sg.detach(), hg.detach(), eps=1e-6)
+    assert O.compare_bf16_ulp(other.cpu(), want.detach()).frac_exact < 0.9 if dtype == torch.bfloat16 else True
+
+
+@pytest.mark.parametrize("cls_name", ["FusedAdaLayerNormZero", "FusedAdaLayerNormZeroSingle"])
+def test_adaln_zero_fp32_layer_norm_fused_vs_eager_branch(FL, gpu_device, cls_name):
+    """The modules built with norm_type="fp32_layer_norm": the fused branch stands in for FP32LayerNorm
+    (eps 1e-5) and must agree with the eager branch, forward and backward, on small-variance rows where the
+    eps is visible."""
+    torch.manual_seed(3)
+    B, S, C = 2, 130, 3072
+    cls = getattr(FL, cls_name)
+    x = (0.02 * torch.randn(B, S, C, device=gpu_device)).bfloat16()
+    temb = torch.randn(B, C, device=gpu_device).bfloat16()
+    g = torch.randn(B, S, C, device=gpu_device).bfloat16()
+    fused = cls(C, norm_type="fp32_layer_norm", fused_kernels=True, linear_parallel=False).to(gpu_device).bfloat16()
+    eager = cls(C, norm_type="fp32_layer_norm", fused_kernels=False, linear_parallel=False).to(gpu_device).bfloat16()
+    eager.load_state_dict(fused.state_dict())
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = fused(xa, emb=temb), eager(xb, emb=temb)
+    ya[0].backward(g)
+    yb[0].backward(g)
+    rep = O.compare_bf16_ulp(ya[0].detach().cpu(), yb[0].detach().cpu())
+    assert rep.frac_exact > 0.999, rep
+    assert O.frac_outside(ya[0].detach().cpu(), yb[0].detach().cpu(), 1e-2, 1e-3) < 1e-5
+    assert O.frac_outside(xa.grad.cpu(), xb.grad.cpu(), 1e-2, 1e-3) < 1e-4
+    ga, gb = fused.linear.weight.grad.float().cpu(), eager.linear.weight.grad.float().cpu()
+    assert (ga - gb).abs().max() <= 2e-2 * gb.abs().max()
+
+
+# ------------------------------------------- the gated op across two blocks
+
+def test_two_blocks_chained_through_the_gated_op(FL, gpu_device):
+    """Two transformer blocks' worth of the residual stream (dit_layerspec.py:126-184):
+        x1, m1 = norm1(h) keeping the stream          (AdaLNResidualFunction)
+        h2, m2 = gated residual + norm2                (attention output a1 = f(m1))
+        h3     = h2 + mlp(m2) * gate                   (the block's last update, left to autograd)
+        x3, m3 = norm1 of the NEXT block on h3, h4, m4 = its gated residual + norm2
+    with stand-ins for attention and MLP (fixed elementwise maps), against the same graph written with eager
+    ops on the CPU.  Every fused Function sees the gradient of the stream arrive from the block after it."""
+    B, S, C = 2, 97, 3072
+    gen = torch.Generator().manual_seed(123)
+    bf = torch.bfloat16
+    h0 = torch.randn(B, S, C, generator=gen).to(bf)
+    mods = [(0.3 * torch.randn(B, C, generator=gen)).to(bf) for _ in range(10)]   # per block: s1, b1, g1, s2, b2
+    w_attn = (1 + 0.1 * torch.randn(C, generator=gen)).to(bf)
+    w_mlp = (0.5 * torch.randn(C, generator=gen)).to(bf)
+    g_out = (0.1 * torch.randn(B, S, C, generator=gen)).to(bf)
+
+    def graph(h, ms, wa, wm, fused):
+        outs = None
+        for blk in range(2):
+            s1, b1, g1, s2, b2 = ms[5 * blk:5 * blk + 5]
+            if fused:
+                h, m1 = FL.modulated_layer_norm_keeping_stream(h, s1, b1, EPS)
+            else:
+                m1 = O.eager_adaln(h, s1, b1, EPS)
+            a = torch.tanh(m1) * wa                                         # stand-in for attention
+            if fused:
+                h, m2 = FL.gated_residual_layer_norm(h, a, g1, s2, b2, EPS)
+            else:
+                h, m2 = O.eager_gated_residual_adaln(h, a, g1, s2, b2, EPS)
+            h = h + (m2 * wm) * g1[:, None]                                  # stand-in for the MLP update
+            outs = h
+        return outs
+
+    cpu = [t.clone().requires_grad_(True) for t in [h0] + mods + [w_attn, w_mlp]]
+    out_c = graph(cpu[0], cpu[1:11], cpu[11], cpu[12], fused=False)
+    out_c.backward(g_out)
+    gpu = [t.to(gpu_device).requires_grad_(True) for t in [h0] + mods + [w_attn, w_mlp]]
+    out_g = graph(gpu[0], gpu[1:11], gpu[11], gpu[12], fused=True)
+    out_g.backward(g_out.to(gpu_device))
+    # forward: the stream after two blocks; one-ulp flips of a norm output pass through tanh and the updates
+    assert O.frac_outside(out_g.detach().cpu(), out_c.detach(), 1e-2, 1e-2) <= 1e-4
+    assert O.compare_bf16_ulp(out_g.detach().cpu(), out_c.detach()).frac_exact > 0.98
+    # the gradient of the stream's input has crossed four fused backward kernels
+    gx, gw = gpu[0].grad.cpu(), cpu[0].grad
+    assert O.frac_outside(gx, gw, 2e-2, 2e-2 * float(gw.float().abs().mean())) <= 1e-3
+    for i in range(1, 11):   # modulation gradients [B, C]: column sums over S rows of terms known to an ulp
+        got, want = gpu[i].grad.float().cpu(), cpu[i].grad.float()
+        assert (got - want).abs().max() <= 3e-2 * want.abs().max() + 1e-3, i
+
+
+# ----------------------------------- the QK-norm call site with rotary tables
+
+@pytest.mark.parametrize("n_txt", [0, 7])
+def test_qkv_split_norm_function_with_rotary_tables(FL, gpu_device, n_txt, monkeypatch):
+    """split + transpose + q/k RMSNorm + apply_rotary_emb on the image tokens (dit_attention.py:191-214, :266-273,
+    :435-443) through QKVSplitNormFunction / split_qkv_and_norm, against the same sequence in eager ops."""
+    B, S, H, D = 2, 61, 3, 128
+    gen = torch.Generator().manual_seed(31)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()
+    wq = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    wk = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    gq, gk, gv = (torch.randn(B, H, S, D, generator=gen).bfloat16() for _ in range(3))
+    cos, sin = O.make_rope_tables(S - n_txt, D, seed=3)
+    # eager: the reference's own sequence
+    mc, wqc, wkc = (t.clone().requires_grad_(True) for t in (mixed, wq, wk))
+    q, k, v = torch.split(mc, [D, D, D], dim=3)
+    q = O.eager_qk_norm_rope(q.transpose(1, 2), wqc, cos, sin)
+    k = O.eager_qk_norm_rope(k.transpose(1, 2), wkc, cos, sin)
+    torch.autograd.backward([q, k, v.transpose(1, 2)], [gq, gk, gv])
+    # fused, through the module-level helper with FUSED_KERNELS on
+    monkeypatch.setenv("FUSED_KERNELS", "1")
+    mg = mixed.to(gpu_device).requires_grad_(True)
+    qn, kn = FL.RMSNorm(D).to(gpu_device).bfloat16(), FL.RMSNorm(D).to(gpu_device).bfloat16()
+    with torch.no_grad():
+        qn.weight.copy_(wq)
+        kn.weight.copy_(wk)
+    fq, fk, fv = FL.split_qkv_and_norm(mg, qn, kn, rotary=(cos.to(gpu_device), sin.to(gpu_device)))
+    assert fq.shape == (B, H, S, D) and fq.is_contiguous()
+    torch.autograd.backward([fq, fk, fv], [t.to(gpu_device) for t in (gq, gk, gv)])
+    yq = O.eager_rmsnorm(mixed[..., :D].transpose(1, 2), wq)
+    fwd_ok(fq, q.detach(), O.rope_excuse(yq, q.detach()))
+    assert torch.equal(fv.cpu(), mixed[..., 2 * D:].transpose(1, 2))
+    grad_ok(mg.grad, mc.grad, allow=1e-5)
+    grad_ok(qn.weight.grad, wqc.grad)
+    grad_ok(kn.weight.grad, wkc.grad)
+    # the helper's eager branch (FUSED_KERNELS off) is the same sequence
+    monkeypatch.setenv("FUSED_KERNELS", "0")
+    eq, ek, ev = FL.split_qkv_and_norm(mixed.to(gpu_device), qn, kn, rotary=(cos.to(gpu_device), sin.to(gpu_device)))
+    assert O.frac_outside(eq.detach().cpu(), q.detach(), 1e-2, 1e-2) == 0.0
+    assert O.frac_outside(ek.detach().cpu(), k.detach(), 1e-2, 1e-2) == 0.0

@@ -532,6 +532,57 @@ def test_rmsnorm_strided_qk_view_matches_eager(capi, gpu_device, B, S, H):
         assert torch.equal(dx.contiguous(), dx_dense)
 
 
+# ------------------------------- rotary embedding fused behind the strided QK-norm
+
+@pytest.mark.parametrize("B,S,H,n_rot", [(1, 1001, 24, 1001), (2, 37, 6, 20), (1, 5, 1, 0), (1, 300, 3, 299), (1, 4, 2, 3)])
+def test_rmsnorm_rope_strided_vs_eager(capi, gpu_device, B, S, H, n_rot):
+    """q_layernorm / k_layernorm on the transposed views, then apply_rotary_emb on the first n_rot tokens
+    (dit_attention.py:266-273, :435-443), as one kernel each way, against the eager sequence."""
+    D = 128
+    q_cpu, k_cpu, q_g, k_g = _qkv_views(B, S, H, D, torch.bfloat16, 15, gpu_device)
+    gen = torch.Generator().manual_seed(16)
+    w = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    grad = torch.randn(B, H, S, D, generator=gen).bfloat16()
+    cos, sin = O.make_rope_tables(n_rot, D, seed=S)
+    cos_g, sin_g = cos.to(gpu_device), sin.to(gpu_device)
+    for x_cpu, x_g in ((q_cpu, q_g), (k_cpu, k_g)):
+        want_out, want_dx, want_dw = O.eager_qk_norm_rope_fwd_bwd(x_cpu, w, cos, sin, grad)
+        y = O.eager_rmsnorm(x_cpu, w)
+        out, rstd = capi.rmsnorm_rope_forward_strided(x_g, w.to(gpu_device), cos_g, sin_g, EPS)
+        assert out.is_contiguous() and out.shape == (B, H, S, D)
+        assert_fwd_bf16(out, want_out, O.rope_excuse(y, want_out), "out")
+        # tokens past the table: exactly the plain strided norm; same statistics everywhere
+        plain, rstd_plain = capi.rmsnorm_forward_strided(x_g, w.to(gpu_device), EPS)
+        assert torch.equal(out[:, :, n_rot:], plain[:, :, n_rot:]) and torch.equal(rstd, rstd_plain)
+        dx, dw = capi.rmsnorm_rope_backward_strided(grad.to(gpu_device), x_g, w.to(gpu_device), rstd, cos_g, sin_g)
+        assert dx.shape == x_g.shape
+        assert_grad_bf16(dx, want_dx, "dx", allow=1e-5)
+        assert_grad_bf16(dw, want_dw, "dweight")
+        # the fused backward equals "rotate the gradient back, then the plain backward", bit for bit
+        gy = grad.clone().requires_grad_(False)
+        yl = y.detach().clone().requires_grad_(True)
+        O.eager_qk_norm_rope(x_cpu, w, cos, sin)  # (shape check of the oracle path)
+        rot = (O.apply_rotary_emb_real(yl[:, :, :n_rot], cos, sin) if n_rot else yl[:, :, :0])
+        torch.cat([rot, yl[:, :, n_rot:]], dim=2).backward(gy)
+        dx2, dw2 = capi.rmsnorm_backward_strided(yl.grad.contiguous().to(gpu_device), x_g, w.to(gpu_device), rstd_plain)
+        assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
+
+
+def test_rmsnorm_rope_rejects_other_head_dims_and_bad_tables(capi, gpu_device):
+    x = torch.zeros(1, 2, 8, 3072, dtype=torch.bfloat16, device=gpu_device)
+    w = torch.ones(3072, dtype=torch.bfloat16, device=gpu_device)
+    t = torch.zeros(8, 3072, device=gpu_device)
+    with pytest.raises(capi.NormError) as e:
+        capi.rmsnorm_rope_forward_strided(x, w, t, t, EPS)
+    assert e.value.status == 2                       # head dimension 128 only
+    x = torch.zeros(1, 2, 8, 128, dtype=torch.bfloat16, device=gpu_device)
+    w = torch.ones(128, dtype=torch.bfloat16, device=gpu_device)
+    t = torch.zeros(9, 128, device=gpu_device)       # more table rows than tokens
+    with pytest.raises(capi.NormError) as e:
+        capi.rmsnorm_rope_forward_strided(x, w, t, t, EPS)
+    assert e.value.status == 1
+
+
 def test_rmsnorm_strided_3072_transposed_and_fp32(capi, gpu_device):
     """[S, B, C] activations viewed as [B, S, C] (the blocks transpose between the two layouts)."""
     S, B, C = 301, 2, 3072
@@ -648,4 +699,10 @@ def test_rows_past_two_to_the_31_elements(capi, gpu_device):
     assert_fwd_bf16(out[idx], want_out, None, "rms out")
     dx, dw = capi.rmsnorm_backward(grad[0], x[0], w, rstd)
     assert_grad_bf16(dx[idx], want_dx, "rms dx")
-    assert torch.isfinite(dw.float()).all()
+    # dweight against an independent fp32 reduction of rnd(g * rnd(x * rstd)) in torch, slice by slice
+    want_dw = torch.zeros(C, device=gpu_device)
+    for lo in range(0, rows, 50_000):
+        xs_, gs_, rs_ = x[0, lo:lo + 50_000].float(), grad[0, lo:lo + 50_000], rstd[lo:lo + 50_000]
+        y = (xs_ * rs_[:, None]).bfloat16()
+        want_dw += (gs_ * y).float().sum(0)
+    assert O.frac_outside(dw.cpu(), want_dw.cpu(), 1e-2, 1e-2) == 0.0

@@ -410,3 +410,100 @@ def test_bf16_ulp_comparator():
     a = torch.tensor([1.0, 1.0, -1.0, 0.0, 2.0 ** -126]).bfloat16()
     b = torch.tensor([1.0078125, 1.015625, -1.0078125, -0.0, 0.0]).bfloat16()
     assert O.bf16_ulp_distance(a, b).tolist() == [1, 2, 1, 0, 128]
+
+
+# ------------------------------------------------- rotary embedding (restated)
+# apply_rotary_emb_real restates a third-party routine (diffusers 0.32.1, absent here).  What follows pins the
+# restatement by what a rotation of adjacent pairs must satisfy; none of it re-types its formula.
+
+def _angles(S, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    th = (torch.rand(S, D // 2, generator=g, dtype=torch.float64) - 0.5) * 12.0
+    rep = lambda t: t.repeat_interleave(2, dim=1)
+    return th, rep(th.cos()).float(), rep(th.sin()).float()
+
+
+def test_rotary_identity_at_angle_zero_is_bit_exact():
+    x = torch.randn(2, 3, 5, 16, generator=torch.Generator().manual_seed(1))
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        xt = x.to(dtype)
+        out = O.apply_rotary_emb_real(xt, torch.ones(5, 16), torch.zeros(5, 16))
+        assert out.dtype == dtype and torch.equal(out, xt)
+
+
+def test_rotary_is_a_complex_multiplication_per_pair_brute_force():
+    B, H, S, D = 2, 2, 3, 8
+    x = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(2), dtype=torch.float64)
+    th, cos, sin = _angles(S, D, 3)
+    got = O.apply_rotary_emb_real(x.float(), cos, sin).double()
+    for b in range(B):
+        for h in range(H):
+            for s in range(S):
+                for i in range(D // 2):
+                    z = complex(x[b, h, s, 2 * i], x[b, h, s, 2 * i + 1]) * complex(math.cos(th[s, i]), math.sin(th[s, i]))
+                    assert abs(got[b, h, s, 2 * i] - z.real) < 1e-5 and abs(got[b, h, s, 2 * i + 1] - z.imag) < 1e-5
+
+
+def test_rotary_preserves_pair_norms_and_composes_angles():
+    B, H, S, D = 1, 2, 7, 32
+    x = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(4))
+    th1, c1, s1 = _angles(S, D, 5)
+    th2, c2, s2 = _angles(S, D, 6)
+    y = O.apply_rotary_emb_real(x, c1, s1)
+    pair = lambda t: t.reshape(B, H, S, D // 2, 2).pow(2).sum(-1)
+    torch.testing.assert_close(pair(y), pair(x), rtol=1e-5, atol=1e-6)
+    rep = lambda t: t.repeat_interleave(2, dim=1).float()
+    both = O.apply_rotary_emb_real(x, rep((th1 + th2).cos()), rep((th1 + th2).sin()))
+    torch.testing.assert_close(O.apply_rotary_emb_real(y, c2, s2), both, rtol=1e-4, atol=1e-5)
+    # a quarter turn maps (a, b) to (-b, a): fixes the direction of rotation and which element is "real"
+    q = O.apply_rotary_emb_real(x, torch.zeros(S, D), torch.ones(S, D))
+    assert torch.equal(q[..., 0::2], -x[..., 1::2]) and torch.equal(q[..., 1::2], x[..., 0::2])
+
+
+def test_rotary_other_conventions_are_visibly_different():
+    B, H, S, D = 1, 1, 4, 16
+    x = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(7))
+    _, cos, sin = _angles(S, D, 8)
+    want = O.apply_rotary_emb_real(x, cos, sin)
+    a, b = x[..., 0::2], x[..., 1::2]
+    clockwise = torch.stack([b, -a], dim=-1).flatten(3)                 # rotate_pairs with the sign on the other element
+    assert (x * cos + clockwise * sin - want).abs().max() > 0.1
+    h1, h2 = x[..., : D // 2], x[..., D // 2:]                          # halves instead of adjacent pairs (unbind dim -2)
+    halves = torch.cat([-h2, h1], dim=-1)
+    assert (x * cos + halves * sin - want).abs().max() > 0.1
+
+
+def test_rotary_gradient_is_the_inverse_rotation():
+    B, H, S, D = 1, 2, 3, 8
+    th, cos, sin = _angles(S, D, 9)
+    x = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(10)).requires_grad_(True)
+    g = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(11))
+    O.apply_rotary_emb_real(x, cos, sin).backward(g)
+    rep = lambda t: t.repeat_interleave(2, dim=1).float()
+    torch.testing.assert_close(x.grad, O.apply_rotary_emb_real(g, rep(th.cos()), rep((-th).sin())), rtol=1e-5, atol=1e-6)
+    # (the map is linear in x, so its gradient is its transpose; for a rotation that is the inverse rotation.
+    # gradcheck does not apply: the routine computes in float32 whatever the input type.)
+    u = torch.randn(B, H, S, D, generator=torch.Generator().manual_seed(12))
+    lhs = (O.apply_rotary_emb_real(u, cos, sin) * g).sum()
+    rhs = (u * x.grad).sum()
+    torch.testing.assert_close(lhs, rhs, rtol=1e-4, atol=1e-4)                  # <R u, g> = <u, R^T g>
+
+
+def test_qk_norm_rope_composition_and_partial_rotation():
+    B, H, S, D, n = 1, 3, 9, 128, 6
+    d = O.make_rmsnorm_inputs((B, H, S), D, torch.bfloat16, seed=12)
+    cos, sin = O.make_rope_tables(n, D, seed=1)
+    assert cos.shape == (n, D) and torch.equal(cos[:, 0::2], cos[:, 1::2])          # one angle per pair
+    torch.testing.assert_close(cos * cos + sin * sin, torch.ones(n, D), rtol=1e-6, atol=1e-6)
+    out, dx, dw = O.eager_qk_norm_rope_fwd_bwd(d["x"], d["weight"], cos, sin, d["grad"])
+    y = O.eager_rmsnorm(d["x"], d["weight"])
+    assert torch.equal(out[:, :, n:], y[:, :, n:])                                   # text tokens: norm only
+    assert torch.equal(out[:, :, :n], O.apply_rotary_emb_real(y[:, :, :n], cos, sin))
+    t_out, t_dx, t_dw = O.truth_qk_norm_rope_fwd_bwd(d["x"], d["weight"], cos, sin, d["grad"])
+    assert (out.double() - t_out).abs().max() < 0.05
+    assert O.frac_outside(dx, t_dx.float(), 3e-2, 3e-2) == 0.0
+    assert O.frac_outside(dw, t_dw.float(), 3e-2, 0.1) == 0.0
+    # no rotation at all (n = 0 tokens) is the plain norm, gradient included
+    o0, dx0, dw0 = O.eager_qk_norm_rope_fwd_bwd(d["x"], d["weight"], cos[:0], sin[:0], d["grad"])
+    p0 = O.eager_rmsnorm_fwd_bwd(d["x"], d["weight"], d["grad"])
+    assert torch.equal(o0, p0[0]) and torch.equal(dx0, p0[1]) and torch.equal(dw0, p0[2])
