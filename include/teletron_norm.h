@@ -187,6 +187,20 @@ int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, co
                       int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                       void *workspace, size_t workspace_bytes, void *stream);
 
+/* tt_adaln_forward / tt_adaln_backward on sequence-first rows: x, out, dout and dx are
+ * [rows_per_sample, batch, cols] (the layout of the blocks' callers; the output norm broadcasts its
+ * per-sample modulation over it, teletron/models/dit/dit_layerspec.py:72-78): sample b owns rows
+ * b, b + batch, ...  mean and rstd are indexed by the same row numbers.  Same scratch as
+ * tt_adaln_backward.  batch * cols * element size must not exceed 256 MiB. */
+int tt_adaln_forward_seq_first(void *out, float *mean, float *rstd, const void *x,
+                               const void *scale, const void *shift,
+                               int64_t batch, int64_t rows_per_sample, int64_t cols,
+                               double eps, int dtype, void *stream);
+int tt_adaln_backward_seq_first(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                                const void *scale, const float *mean, const float *rstd,
+                                int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
 /* tt_adaln_backward without a scratch argument, for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
  * no counterpart in the reference.  The partial column sums go to a static device array of

@@ -27,6 +27,7 @@ EXPORTS = (
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
     "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual", "tt_adaln_backward_static",
     "tt_norm_stream_probe", "tt_rmsnorm_rope_forward_strided", "tt_rmsnorm_rope_backward_strided",
+    "tt_adaln_forward_seq_first", "tt_adaln_backward_seq_first",
 )
 
 
@@ -66,6 +67,8 @@ def lib() -> ctypes.CDLL:
         L.tt_adaln_backward_workspace_bytes.restype = sz
         L.tt_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
         L.tt_adaln_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
+        L.tt_adaln_forward_seq_first.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, dbl, ci, vp]
+        L.tt_adaln_backward_seq_first.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_static.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.tt_adaln_backward_from_xnorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp, sz, vp]
         L.tt_gated_residual_adaln_forward.argtypes = [vp] * 9 + [i64, i64, i64, dbl, ci, vp]
@@ -224,8 +227,8 @@ def rmsnorm_rope_backward_strided(dout, x, weight, rstd, cos, sin, dx=None):
     return dx, dweight
 
 
-def adaln_forward(x, scale, shift, eps: float, want_xnorm: bool = False):
-    """x [B, S, C] (or [rows, C] with scale [1, C]); returns (out, mean, rstd) or
+def adaln_forward(x, scale, shift, eps: float, want_xnorm: bool = False, seq_first: bool = False):
+    """x [B, S, C] (or [rows, C] with scale [1, C]; [S, B, C] with seq_first); returns (out, mean, rstd) or
     (out, x_norm, rstd) when want_xnorm."""
     _dense_gpu(x, scale, shift)
     cols = x.shape[-1]
@@ -243,12 +246,13 @@ def adaln_forward(x, scale, shift, eps: float, want_xnorm: bool = False):
                    "tt_adaln_forward_xnorm")
             return out, xn, rstd
         mean = torch.empty(rows, dtype=torch.float32, device=x.device)
-        _check(lib().tt_adaln_forward(_p(out), _p(mean), _p(rstd), _p(x), _p(scale), _p(shift), batch,
-                                      rows // batch, cols, eps, _dt(x), _stream(x)), "tt_adaln_forward")
+        fn = lib().tt_adaln_forward_seq_first if seq_first else lib().tt_adaln_forward
+        _check(fn(_p(out), _p(mean), _p(rstd), _p(x), _p(scale), _p(shift), batch,
+                  rows // batch, cols, eps, _dt(x), _stream(x)), "tt_adaln_forward")
     return out, mean, rstd
 
 
-def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False):
+def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False, seq_first: bool = False):
     _dense_gpu(dout, x, scale, rstd)
     cols = x.shape[-1]
     batch = scale.numel() // cols
@@ -265,8 +269,9 @@ def adaln_backward(dout, x, scale, mean, rstd, from_xnorm: bool = False):
                                                   _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n,
                                                   _stream(x)), "tt_adaln_backward_from_xnorm")
         else:
-            _check(L.tt_adaln_backward(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(x), _p(scale), _p(mean),
-                                       _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n, _stream(x)),
+            fn = L.tt_adaln_backward_seq_first if seq_first else L.tt_adaln_backward
+            _check(fn(_p(dx), _p(dscale), _p(dshift), _p(dout), _p(x), _p(scale), _p(mean),
+                      _p(rstd), batch, rows // batch, cols, _dt(x), _p(ws), n, _stream(x)),
                    "tt_adaln_backward")
     return dx, dscale, dshift
 

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     T *__restrict__ out, T *__restrict__ xnorm, float *__restrict__ mean, float *__restrict__ rstd,
     const T *__restrict__ x, const T *__restrict__ scale, const T *__restrict__ shift,
     T *__restrict__ h2_out, const T *__restrict__ attn, const T *__restrict__ gate,
-    int64_t rows_per_sample, int blocks_per_sample, float eps) {
+    int64_t rows_per_sample, const SampleLayout lay, int blocks_per_sample, float eps) {
     using G = RowGeom<T, C>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, LANES = G::LANES, CHUNKS = G::CHUNKS, RPW = G::RPW;
@@ -129,10 +129,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         keep_packed(hr);
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         const bool ok = rs < rows_per_sample;
-        const int64_t row = b * rows_per_sample + rs;
-        // the wavefront's rows are consecutive: where it writes starts at its first row
-        const int64_t first = (b * rows_per_sample + grp * RPW) * C;
-        const uint32_t lane_bytes = (uint32_t)((sub * C) * sizeof(T)) + l * 16;
+        const int64_t row = lay.row(b, rs);
+        // where the wavefront writes starts at its first row; the lane adds the distance to its own row
+        const int64_t first = lay.row(b, grp * RPW) * C;
+        const uint32_t lane_bytes = (uint32_t)(sub * lay.row_stride * C * sizeof(T)) + l * 16;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(x + row * C) + l;
         u32x4 xr[CHUNKS];
 #pragma unroll
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const T *__restrict__ xin, const T *__restrict__ scale, const float *__restrict__ mean,
     const float *__restrict__ rstd, T *__restrict__ da, const T *__restrict__ e,
     const T *__restrict__ attn, const T *__restrict__ gate, int64_t rows_per_sample,
-    int blocks_per_sample) {
+    const SampleLayout lay, int blocks_per_sample) {
     static_assert(!(GATED && FROM_XNORM), "the gated form works from the saved h2");
     static_assert(!(GATED && RES), "the gated form handles e itself");
     constexpr int NSETS = GATED ? 3 : 2;
@@ -299,8 +299,8 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     auto fetch = [&](RowRegs &b, int64_t grp) {
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         b.ok = rs < rows_per_sample;
-        b.row = smp * rows_per_sample + rs;
-        b.first = (smp * rows_per_sample + grp * RPW) * C;
+        b.row = lay.row(smp, rs);
+        b.first = lay.row(smp, grp * RPW) * C;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
 #if TTN_BWD_LOAD_RUNS
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         const float K1 = FROM_XNORM ? k1 : k1 * r;
         const float K0 = FROM_XNORM ? k0 : fmaf(k1, nmr, k0);
 
-        const uint32_t lane_bytes = (uint32_t)((sub * C) * sizeof(T)) + l * 16;
+        const uint32_t lane_bytes = (uint32_t)(sub * lay.row_stride * C * sizeof(T)) + l * 16;
         constexpr int kDxStore = (GATED ? 0 : TTN_ADALN_BWD_STORE);
         const RowWriter<kDxStore> wd(dx + b.first, lane_bytes);
         const RowWriter<0> wa(GATED ? da + b.first : nullptr, lane_bytes);
@@ -482,6 +482,10 @@ struct AdalnArgs {
     int64_t batch, rows_per_sample;
     double eps;
     hipStream_t stream;
+    bool seq_first = false;  // rows laid out [rows_per_sample, batch] instead of [batch, rows_per_sample]
+    SampleLayout layout() const {
+        return seq_first ? SampleLayout{1, batch} : SampleLayout{rows_per_sample, 1};
+    }
 };
 
 struct GatedPtrs {  // the extra operands of the gated-residual form (all null otherwise)
@@ -506,8 +510,8 @@ static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, con
         RowKernelProfile prof(a.stream);
         adaln_fwd_kernel<T, C, WRITE_XNORM, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), TTN_ADALN_FWD_DYN_LDS, a.stream>>>(
             (T *)out, (T *)xnorm, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift,
-            (T *)gp.h2_or_da, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample, p.blocks_per_sample,
-            (float)a.eps);
+            (T *)gp.h2_or_da, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample, a.layout(),
+            p.blocks_per_sample, (float)a.eps);
     }
     return check_launch("adaln forward launch");
 }
@@ -539,7 +543,7 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
         adaln_bwd_kernel<T, C, FROM_XNORM, GATED, RES><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(
             (T *)dx, (float *)ws, (const T *)g, (const T *)xin, (const T *)scale, mean, rstd,
             (T *)gp.h2_or_da, (const T *)gp.e, (const T *)gp.attn, (const T *)gp.gate, a.rows_per_sample,
-            p.blocks_per_sample);
+            a.layout(), p.blocks_per_sample);
     }
     st = check_launch("adaln backward launch");
     if (st != TT_NORM_OK) return st;
@@ -565,6 +569,19 @@ static int check_adaln_args(const char *who, int64_t batch, int64_t rows_per_sam
         if (!p) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
         if (!aligned16(p)) return fail(TT_NORM_EALIGN, "%s: pointer %p not 16-byte aligned", who, p);
     }
+    return TT_NORM_OK;
+}
+
+static int wide_form_unsupported(const char *who, int64_t cols) {
+    return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld (this form takes 3072 columns, or any row of up to 384 16-byte "
+                "pieces: 3072 two-byte / 1536 four-byte columns)", who, (long long)cols);
+}
+
+// The rows a wavefront handles together (up to eight when rows are narrow) are addressed with 32-bit
+// byte offsets from the first of them; in the sequence-first layout they lie batch rows apart.
+static int check_seq_first(const char *who, int64_t batch, int64_t cols, int dtype) {
+    if (batch * cols * (int64_t)elem_bytes(dtype) > (int64_t)(1 << 28))
+        return fail(TT_NORM_EINVAL, "%s: batch * cols * element size exceeds 256 MiB", who);
     return TT_NORM_OK;
 }
 
@@ -664,6 +681,44 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
 #undef CALL
 }
 
+/* ---- sequence-first rows: x is [rows_per_sample, batch, cols] ---- */
+
+int tt_adaln_forward_seq_first(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                               const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                               double eps, int dtype, void *stream) {
+    int st = check_adaln_args("tt_adaln_forward_seq_first", batch, rows_per_sample, cols, dtype, {out, x, scale, shift});
+    if (st == TT_NORM_OK) st = check_seq_first("tt_adaln_forward_seq_first", batch, cols, dtype);
+    if (st != TT_NORM_OK) return st;
+    if ((!mean || !rstd) && rows_per_sample > 0) return fail(TT_NORM_EINVAL, "tt_adaln_forward_seq_first: null mean/rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_adaln_forward(out, mean, rstd, x, scale, shift, batch, rows_per_sample, cols, eps, dtype,
+                                      (hipStream_t)stream, true);
+    const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream, true};
+#define CALL(T, C) return adaln_forward_t<T, C, false>(out, nullptr, mean, rstd, x, scale, shift, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
+int tt_adaln_backward_seq_first(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
+                                const void *scale, const float *mean, const float *rstd, int64_t batch,
+                                int64_t rows_per_sample, int64_t cols, int dtype, void *workspace,
+                                size_t workspace_bytes, void *stream) {
+    int st = check_adaln_args("tt_adaln_backward_seq_first", batch, rows_per_sample, cols, dtype, {dx, dout, x, scale});
+    if (st == TT_NORM_OK) st = check_seq_first("tt_adaln_backward_seq_first", batch, cols, dtype);
+    if (st != TT_NORM_OK) return st;
+    if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
+        return fail(TT_NORM_EINVAL, "tt_adaln_backward_seq_first: null dscale/dshift/mean/rstd");
+    if (!tuned_shape(cols, dtype))
+        return anywidth_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols,
+                                       dtype, workspace, workspace_bytes, (hipStream_t)stream, true);
+    const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream, true};
+#define CALL(T, C)                                                                                \
+    return adaln_backward_t<T, C, false>(dx, dscale, dshift, dout, x, scale, mean, rstd, dtype, workspace, \
+                                         workspace_bytes, a)
+    TTN_DISPATCH(dtype, cols, CALL);
+#undef CALL
+}
+
 /* ---- AdaLN backward that allocates nothing: scratch in a static device array ---- */
 
 }  // extern "C"
@@ -726,11 +781,15 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
                                     const void *shift, int64_t batch, int64_t rows_per_sample,
                                     int64_t cols, double eps, int dtype, void *stream) {
     int st = check_adaln_args("tt_gated_residual_adaln_forward", batch, rows_per_sample, cols, dtype,
-                              {h2, out, h, attn, gate, scale, shift}, true);
+                              {h2, out, h, attn, gate, scale, shift});
     if (st != TT_NORM_OK) return st;
-    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_forward: built for cols 3072 only");
     if ((!mean || !rstd) && rows_per_sample > 0)
         return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_forward: null mean/rstd");
+    if (cols != 3072) {
+        if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_gated_residual_adaln_forward", cols);
+        return anywidth_gated_adaln_forward(h2, out, mean, rstd, h, attn, gate, scale, shift, batch, rows_per_sample, cols,
+                                            eps, dtype, (hipStream_t)stream);
+    }
     const AdalnArgs a{batch, rows_per_sample, eps, (hipStream_t)stream};
     const GatedPtrs gp{h2, nullptr, attn, gate};
     if (dtype == TT_NORM_BF16)
@@ -742,6 +801,7 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
 
 size_t tt_gated_residual_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols,
                                                         int dtype) {
+    if (cols != 3072 && !anywidth_wide_forms_supported(cols, dtype)) return 0;
     // three sets of column sums (dscale, dshift, dgate) instead of two
     return tt_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype) / 2 * 3;
 }
@@ -753,12 +813,17 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                      int64_t cols, int dtype, void *workspace, size_t workspace_bytes,
                                      void *stream) {
     int st = check_adaln_args("tt_gated_residual_adaln_backward", batch, rows_per_sample, cols, dtype,
-                              {dh, dattn, dout, h2, attn, gate, scale}, true);
+                              {dh, dattn, dout, h2, attn, gate, scale});
     if (st != TT_NORM_OK) return st;
-    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_gated_residual_adaln_backward: built for cols 3072 only");
     if (dh2 && !aligned16(dh2)) return fail(TT_NORM_EALIGN, "tt_gated_residual_adaln_backward: dh2 not 16-byte aligned");
     if (!dgate || !dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_backward: null dgate/dscale/dshift/mean/rstd");
+    if (cols != 3072) {
+        if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_gated_residual_adaln_backward", cols);
+        return anywidth_gated_adaln_backward(dh, dattn, dgate, dscale, dshift, dout, dh2, h2, attn, gate, scale, mean, rstd,
+                                             batch, rows_per_sample, cols, dtype, workspace, workspace_bytes,
+                                             (hipStream_t)stream);
+    }
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
     const GatedPtrs gp{dattn, dh2, attn, gate};
     if (dtype == TT_NORM_BF16)
@@ -778,11 +843,15 @@ int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void 
                                int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                void *workspace, size_t workspace_bytes, void *stream) {
     int st = check_adaln_args("tt_adaln_backward_residual", batch, rows_per_sample, cols, dtype,
-                              {dx, dout, dres, x, scale}, true);
+                              {dx, dout, dres, x, scale});
     if (st != TT_NORM_OK) return st;
-    if (cols != 3072) return fail(TT_NORM_EUNSUPPORTED, "tt_adaln_backward_residual: built for cols 3072 only");
     if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward_residual: null dscale/dshift/mean/rstd");
+    if (cols != 3072) {
+        if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_adaln_backward_residual", cols);
+        return anywidth_adaln_backward_residual(dx, dscale, dshift, dout, dres, x, scale, mean, rstd, batch, rows_per_sample,
+                                                cols, dtype, workspace, workspace_bytes, (hipStream_t)stream);
+    }
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
     const GatedPtrs gp{nullptr, dres, nullptr, nullptr};
     if (dtype == TT_NORM_BF16)

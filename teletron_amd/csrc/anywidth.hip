@@ -101,10 +101,10 @@ __device__ __forceinline__ void flush_partials_anywidth(float (&acc)[NSETS][G::C
 
 // ------------------------------------------------------------------ RMSNorm
 
-template <typename T, int LANES, int CHUNKS>
+template <typename T, int LANES, int CHUNKS, typename Map>
 __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
     T *__restrict__ out, float *__restrict__ rstd, const T *__restrict__ x, const T *__restrict__ w,
-    int64_t rows, int C, float eps) {
+    const Map map, int C, float eps) {
     using G = PadGeom<T, LANES, CHUNKS>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, RPW = G::RPW;
@@ -117,14 +117,15 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
     u32x4 wr[CHUNKS];
     load_param<G>(wr, w, l, m);
 
-    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t groups = map.template groups<RPW>();
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
         keep_packed(wr);
-        const int64_t row = grp * RPW + sub;
-        const bool ok = row < rows;
+        const RowAddr at = map.template locate<RPW>(grp, sub, C);
+        const int64_t row = at.row;
+        const bool ok = at.ok;
         u32x4 xr[CHUNKS];
-        load_row<G>(xr, x + row * C, l, ok, m);
+        load_row<G>(xr, x + at.xoff, l, ok, m);
 
         float ss = 0.0f;
 #pragma unroll
@@ -138,7 +139,9 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
         const float r = 1.0f / sqrtf(ss / (float)C + eps);
         if (ok && l == 0) rstd[row] = r;
 
-        const RowWriter<TTN_ANY_FWD_STORE> wo(out + grp * RPW * C, (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
+        // the wavefront's rows are consecutive in out: base = its first row
+        const RowWriter<TTN_ANY_FWD_STORE> wo(out + map.template locate<RPW>(grp, 0, C).row * C,
+                                              (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], wv[VEC];
@@ -154,10 +157,10 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_fwd_kernel(
     }
 }
 
-template <typename T, int LANES, int CHUNKS>
+template <typename T, int LANES, int CHUNKS, typename Map>
 __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g, const T *__restrict__ x,
-    const T *__restrict__ w, const float *__restrict__ rstd, int64_t rows, int C) {
+    const T *__restrict__ w, const float *__restrict__ rstd, const Map map, int C) {
     using G = PadGeom<T, LANES, CHUNKS>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, RPW = G::RPW;
@@ -176,15 +179,16 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[0][k][j] = 0.0f;
 
-    const int64_t groups = (rows + RPW - 1) / RPW;
+    const int64_t groups = map.template groups<RPW>();
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
         keep_packed(wr);
-        const int64_t row = grp * RPW + sub;
-        const bool ok = row < rows;
+        const RowAddr at = map.template locate<RPW>(grp, sub, C);
+        const int64_t row = at.row;
+        const bool ok = at.ok;
         u32x4 gr[CHUNKS], xr[CHUNKS];
         load_row<G>(gr, g + row * C, l, ok, m);
-        load_row<G>(xr, x + row * C, l, ok, m);
+        load_row<G>(xr, x + at.xoff, l, ok, m);
         const float r = ok ? rstd[row] : 0.0f;
 
         // pass 1: gy = rnd(g*w) kept packed; row dot  sum_c gy * x
@@ -211,8 +215,10 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
         keep_packed(xr);
         keep_packed(gyp);
 
-        const RowWriter<(TTN_ANY_BWD_STORE && CHUNKS <= 6)> wd(dx + grp * RPW * C,
-                                                               (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
+        // dx goes through its own strides: base = the wavefront's first row, the lane adds its row's distance
+        const int64_t doff0 = map.template locate<RPW>(grp, 0, C).doff;
+        const RowWriter<(TTN_ANY_BWD_STORE && CHUNKS <= 6)> wd(
+            dx + doff0, (uint32_t)((at.doff - doff0) * (int64_t)sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
@@ -238,11 +244,14 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_rmsnorm_bwd_kernel(
 
 // -------------------------------------------------------------------- AdaLN
 
-template <typename T, int LANES, int CHUNKS>
+// GATED = true: the normalised row is first formed as h2 = rnd(x + rnd(attn * gate[b])) (the gated residual
+// update that precedes the norm in the transformer blocks) and written out too.
+template <typename T, int LANES, int CHUNKS, bool GATED>
 __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
     T *__restrict__ out, float *__restrict__ mean, float *__restrict__ rstd, const T *__restrict__ x,
-    const T *__restrict__ scale, const T *__restrict__ shift, int64_t rows_per_sample, int blocks_per_sample,
-    int C, float eps) {
+    const T *__restrict__ scale, const T *__restrict__ shift, T *__restrict__ h2_out, const T *__restrict__ attn,
+    const T *__restrict__ gate, int64_t rows_per_sample, const SampleLayout lay, int blocks_per_sample, int C,
+    float eps) {
     using G = PadGeom<T, LANES, CHUNKS>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, RPW = G::RPW;
@@ -255,8 +264,10 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
     const LaneMask<G> m(l, C / VEC);
 
     u32x4 tr[CHUNKS], hr[CHUNKS];
+    [[maybe_unused]] u32x4 qr[GATED ? CHUNKS : 1];
     load_param<G>(tr, scale + b * C, l, m);
     load_param<G>(hr, shift + b * C, l, m);
+    if constexpr (GATED) load_param<G>(qr, gate + b * C, l, m);
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) {  // t = rnd(1 + scale)
         float v[VEC];
@@ -271,11 +282,33 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
     for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
         keep_packed(tr);
         keep_packed(hr);
+        if constexpr (GATED) keep_packed(qr);
         const int64_t rs = grp * RPW + sub;
         const bool ok = rs < rows_per_sample;
-        const int64_t row = b * rows_per_sample + rs;
+        const int64_t row = lay.row(b, rs);
+        const int64_t first = lay.row(b, grp * RPW) * C;  // the wavefront's first row: base of what it writes
+        const uint32_t lane_bytes = (uint32_t)(sub * lay.row_stride * C * (int64_t)sizeof(T)) + l * 16;
         u32x4 xr[CHUNKS];
         load_row<G>(xr, x + row * C, l, ok, m);
+        if constexpr (GATED) {
+            u32x4 ar[CHUNKS];
+            load_row<G>(ar, attn + row * C, l, ok, m);
+            const RowWriter<TTN_ANY_FWD_STORE> wh(h2_out + first, lane_bytes);
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+                float hv[VEC], av[VEC], gv[VEC];
+                E::unpack(xr[k], hv);
+                E::unpack(ar[k], av);
+                E::unpack(qr[k], gv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) av[j] *= gv[j];
+                E::round(av);  // attn * gate materialised in the element type
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) hv[j] += av[j];
+                xr[k] = E::pack(hv);  // h2: the new residual stream, and the row that is normalised
+                if (ok && m.in[k]) wh.put(k * LANES, xr[k]);
+            }
+        }
 
         float s = 0.0f;
 #pragma unroll
@@ -306,8 +339,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
         }
 
         const float nmr = -(mu * r);
-        const RowWriter<TTN_ANY_FWD_STORE> wo(out + (b * rows_per_sample + grp * RPW) * C,
-                                              (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
+        const RowWriter<TTN_ANY_FWD_STORE> wo(out + first, lane_bytes);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], tv[VEC], hv[VEC];
@@ -327,11 +359,19 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_fwd_kernel(
     }
 }
 
-template <typename T, int LANES, int CHUNKS>
+// GATED: x is the saved h2; dx = dh = rnd(rnd(dx of the norm) + e) with e the gradient arriving at h2 from
+// its other use (may be null), da = rnd(dh * gate[b]) is written too and dgate[b] += rnd(dh * attn) is a
+// third set of column sums.  RES: dx = rnd(rnd(dx of the norm) + e), e the gradient the input receives
+// from its other consumer.  (Same forms as the tuned kernels.)
+template <typename T, int LANES, int CHUNKS, bool GATED, bool RES>
 __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
     T *__restrict__ dx, float *__restrict__ partial, const T *__restrict__ g, const T *__restrict__ x,
     const T *__restrict__ scale, const float *__restrict__ mean, const float *__restrict__ rstd,
-    int64_t rows_per_sample, int blocks_per_sample, int C) {
+    T *__restrict__ da, const T *__restrict__ e, const T *__restrict__ attn, const T *__restrict__ gate,
+    int64_t rows_per_sample, const SampleLayout lay, int blocks_per_sample, int C) {
+    static_assert(!(GATED && RES), "the gated form handles e itself");
+    static_assert(!(GATED || RES) || CHUNKS <= 6, "the gated and residual forms are built for rows of up to six accesses per lane");
+    constexpr int NSETS = GATED ? 3 : 2;
     using G = PadGeom<T, LANES, CHUNKS>;
     using E = Elem<T>;
     constexpr int VEC = G::VEC, RPW = G::RPW;
@@ -357,6 +397,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
         return E::pack(v);
     };
     u32x4 tr[kParamInRegs ? CHUNKS : 1];
+    [[maybe_unused]] u32x4 qr[GATED ? CHUNKS : 1];
     u32x4 *lds_t = reinterpret_cast<u32x4 *>(lds);  // shares the flush area: dead before the flush starts
     if constexpr (kParamInRegs) {
         load_param<G>(tr, scale + b * C, l, m);
@@ -367,10 +408,11 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
             lds_t[i] = one_plus(load16(reinterpret_cast<const u32x4 *>(scale + b * C) + i));
         __syncthreads();
     }
+    if constexpr (GATED) load_param<G>(qr, gate + b * C, l, m);
 
-    float acc[2][CHUNKS][VEC];  // [0] = dscale, [1] = dshift
+    float acc[NSETS][CHUNKS][VEC];  // [0] = dscale, [1] = dshift, [2] = dgate
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < NSETS; ++s)
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
@@ -380,12 +422,18 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
     for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
         if constexpr (kParamInRegs) keep_packed(tr);
+        if constexpr (GATED) keep_packed(qr);
         const int64_t rs = grp * RPW + sub;
         const bool ok = rs < rows_per_sample;
-        const int64_t row = b * rows_per_sample + rs;
+        const int64_t row = lay.row(b, rs);
+        const int64_t first = lay.row(b, grp * RPW) * C;
+        const uint32_t lane_bytes = (uint32_t)(sub * lay.row_stride * C * (int64_t)sizeof(T)) + l * 16;
         u32x4 gr[CHUNKS], xr[CHUNKS];
+        [[maybe_unused]] u32x4 er[(GATED || RES) ? CHUNKS : 1], ar[GATED ? CHUNKS : 1];
         load_row<G>(gr, g + row * C, l, ok, m);
         load_row<G>(xr, x + row * C, l, ok, m);
+        if constexpr (GATED || RES) load_row<G>(er, e + row * C, l, ok && e != nullptr, m);
+        if constexpr (GATED) load_row<G>(ar, attn + row * C, l, ok, m);
         const float r = ok ? rstd[row] : 0.0f;
         const float mu = ok ? mean[row] : 0.0f;
         const float nmr = -(mu * r);  // xhat = x*r + nmr
@@ -440,8 +488,9 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
         keep_packed(xr);
         if constexpr (kKeepGx) keep_packed(gxp);
 
-        const RowWriter<(TTN_ANY_BWD_STORE && CHUNKS <= 6)> wd(dx + (b * rows_per_sample + grp * RPW) * C,
-                                                               (uint32_t)(sub * C * (int)sizeof(T)) + l * 16);
+        constexpr int kDxStore = (TTN_ANY_BWD_STORE && CHUNKS <= 6 && !GATED);
+        const RowWriter<kDxStore> wd(dx + first, lane_bytes);
+        const RowWriter<0> wa(GATED ? da + first : nullptr, lane_bytes);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
@@ -457,7 +506,30 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
                 xn[j] = centred<T>(xv[j], mu, r, nmr);
                 acc[1][k][j] += gv[j];
             }
-            if (ok && m.in[k]) wd.put(k * LANES, E::pack(o));
+            if constexpr (GATED || RES) {
+                float ev[VEC];
+                E::round(o);  // the norm's dx, materialised in the element type
+                E::unpack(er[k], ev);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o[j] += ev[j];
+            }
+            const u32x4 dxp = E::pack(o);
+            if (ok && m.in[k]) wd.put(k * LANES, dxp);
+            if constexpr (GATED) {
+                float av[VEC], qv[VEC];
+                E::unpack(dxp, o);  // dh as stored
+                E::unpack(ar[k], av);
+                E::unpack(qr[k], qv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    qv[j] *= o[j];
+                    av[j] *= o[j];
+                }
+                if (ok && m.in[k]) wa.put(k * LANES, E::pack(qv));
+                E::round(av);  // dh*attn materialised in the element type before the column sum
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
+            }
             E::round(xn);  // the normalised row in the element type
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
@@ -467,7 +539,7 @@ __global__ __launch_bounds__(kRowThreads) void anywidth_adaln_bwd_kernel(
         }
     }
     if constexpr (!kParamInRegs) __syncthreads();  // every wavefront is done reading lds_t
-    flush_partials_anywidth<G, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), lds, C, m);
+    flush_partials_anywidth<G, NSETS>(acc, partial + (int64_t)blockIdx.x * (NSETS * C), lds, C, m);
 }
 
 // ---------------------------------------------------------------- dispatch
@@ -536,63 +608,97 @@ static int plan_for(RowPlan *plan, int64_t batch, int64_t rows_per_sample, GeomC
     return TT_NORM_OK;
 }
 
-template <typename T, int LANES, int CHUNKS>
-struct RmsFwd {
-    static int run(const RowPlan &p, void *out, float *rstd, const void *x, const void *w, int64_t rows, int C,
-                   double eps, hipStream_t stream) {
-        RowKernelProfile prof(stream);
-        anywidth_rmsnorm_fwd_kernel<T, LANES, CHUNKS><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-            (T *)out, rstd, (const T *)x, (const T *)w, rows, C, (float)eps);
-        return TT_NORM_OK;
-    }
+template <typename Map>
+struct RmsOn {  // the RMSNorm kernels over one kind of row map
+    template <typename T, int LANES, int CHUNKS>
+    struct Fwd {
+        static int run(const RowPlan &p, void *out, float *rstd, const void *x, const void *w, const Map &map, int C,
+                       double eps, hipStream_t stream) {
+            RowKernelProfile prof(stream);
+            anywidth_rmsnorm_fwd_kernel<T, LANES, CHUNKS, Map><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+                (T *)out, rstd, (const T *)x, (const T *)w, map, C, (float)eps);
+            return TT_NORM_OK;
+        }
+    };
+    template <typename T, int LANES, int CHUNKS>
+    struct Bwd {
+        static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *w,
+                       const float *rstd, const Map &map, int C, hipStream_t stream) {
+            RowKernelProfile prof(stream);
+            anywidth_rmsnorm_bwd_kernel<T, LANES, CHUNKS, Map>
+                <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)C * sizeof(float), stream>>>(
+                    (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)w, rstd, map, C);
+            return TT_NORM_OK;
+        }
+    };
 };
 
-template <typename T, int LANES, int CHUNKS>
-struct RmsBwd {
-    static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *w,
-                   const float *rstd, int64_t rows, int C, hipStream_t stream) {
-        RowKernelProfile prof(stream);
-        anywidth_rmsnorm_bwd_kernel<T, LANES, CHUNKS>
-            <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)C * sizeof(float), stream>>>(
-                (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)w, rstd, rows, C);
-        return TT_NORM_OK;
-    }
+struct AdalnExtra {  // operands of the gated / residual forms (null otherwise)
+    void *h2_or_da;   // forward: h2 out; backward: dattn out
+    const void *e;    // backward: the other gradient (dh2 or dres), may be null for the gated form
+    const void *attn;
+    const void *gate;
 };
 
-template <typename T, int LANES, int CHUNKS>
-struct AdalnFwd {
-    static int run(const RowPlan &p, void *out, float *mean, float *rstd, const void *x, const void *scale,
-                   const void *shift, int64_t rows_per_sample, int C, double eps, hipStream_t stream) {
-        RowKernelProfile prof(stream);
-        anywidth_adaln_fwd_kernel<T, LANES, CHUNKS><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
-            (T *)out, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift, rows_per_sample,
-            p.blocks_per_sample, C, (float)eps);
-        return TT_NORM_OK;
-    }
+template <bool GATED, bool RES>
+struct AdalnOn {
+    template <typename T, int LANES, int CHUNKS>
+    struct Fwd {
+        static int run(const RowPlan &p, void *out, float *mean, float *rstd, const void *x, const void *scale,
+                       const void *shift, const AdalnExtra &ex, int64_t rows_per_sample, SampleLayout lay, int C,
+                       double eps, hipStream_t stream) {
+            if constexpr (GATED && CHUNKS > 6) {
+                return fail(TT_NORM_EUNSUPPORTED, "gated residual + AdaLN: rows of more than six 16-byte accesses per lane");
+            } else {
+                RowKernelProfile prof(stream);
+                anywidth_adaln_fwd_kernel<T, LANES, CHUNKS, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
+                    (T *)out, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift, (T *)ex.h2_or_da,
+                    (const T *)ex.attn, (const T *)ex.gate, rows_per_sample, lay, p.blocks_per_sample, C, (float)eps);
+                return TT_NORM_OK;
+            }
+        }
+    };
+    template <typename T, int LANES, int CHUNKS>
+    struct Bwd {
+        static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *scale,
+                       const float *mean, const float *rstd, const AdalnExtra &ex, int64_t rows_per_sample,
+                       SampleLayout lay, int C, hipStream_t stream) {
+            if constexpr ((GATED || RES) && CHUNKS > 6) {
+                return fail(TT_NORM_EUNSUPPORTED, "gated / residual AdaLN backward: rows of more than six 16-byte accesses per lane");
+            } else {
+                constexpr int NSETS = GATED ? 3 : 2;
+                RowKernelProfile prof(stream);
+                anywidth_adaln_bwd_kernel<T, LANES, CHUNKS, GATED, RES>
+                    <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)NSETS * C * sizeof(float), stream>>>(
+                        (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)scale, mean, rstd,
+                        (T *)ex.h2_or_da, (const T *)ex.e, (const T *)ex.attn, (const T *)ex.gate, rows_per_sample,
+                        lay, p.blocks_per_sample, C);
+                return TT_NORM_OK;
+            }
+        }
+    };
 };
 
-template <typename T, int LANES, int CHUNKS>
-struct AdalnBwd {
-    static int run(const RowPlan &p, void *dx, void *ws, const void *g, const void *x, const void *scale,
-                   const float *mean, const float *rstd, int64_t rows_per_sample, int C, hipStream_t stream) {
-        RowKernelProfile prof(stream);
-        anywidth_adaln_bwd_kernel<T, LANES, CHUNKS>
-            <<<dim3((unsigned)p.blocks), dim3(kRowThreads), (size_t)2 * C * sizeof(float), stream>>>(
-                (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)scale, mean, rstd, rows_per_sample,
-                p.blocks_per_sample, C);
-        return TT_NORM_OK;
-    }
-};
-
-int anywidth_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
-                             double eps, int dtype, hipStream_t stream) {
+template <typename Map>
+static int rmsnorm_forward_on(void *out, float *rstd, const void *x, const void *w, const Map &map, int64_t rows,
+                              int64_t cols, double eps, int dtype, hipStream_t stream) {
     if (rows == 0) return TT_NORM_OK;
     const GeomChoice gc = geometry_for(cols, dtype);
     RowPlan p;
     int st = plan_for(&p, 1, rows, gc, false);
     if (st != TT_NORM_OK) return st;
-    st = dispatch<RmsFwd>(dtype, gc, p, out, rstd, x, w, rows, (int)cols, eps, stream);
+    st = dispatch<RmsOn<Map>::template Fwd>(dtype, gc, p, out, rstd, x, w, map, (int)cols, eps, stream);
     return st != TT_NORM_OK ? st : check_launch("rmsnorm forward launch");
+}
+
+int anywidth_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
+                             double eps, int dtype, hipStream_t stream) {
+    return rmsnorm_forward_on(out, rstd, x, w, DenseRows{rows}, rows, cols, eps, dtype, stream);
+}
+
+int anywidth_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void *w, const Strided3Rows &map,
+                                     int64_t cols, double eps, int dtype, hipStream_t stream) {
+    return rmsnorm_forward_on(out, rstd, x, w, map, map.n0 * map.n1 * map.n2, cols, eps, dtype, stream);
 }
 
 static size_t backward_scratch(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, int nsets) {
@@ -606,9 +712,10 @@ size_t anywidth_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int
     return backward_scratch(1, rows, cols, dtype, 1);
 }
 
-int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
-                              const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
-                              size_t ws_bytes, hipStream_t stream) {
+template <typename Map>
+static int rmsnorm_backward_on(void *dx, void *dw, const void *g, const void *x, const void *w, const float *rstd,
+                               const Map &map, int64_t rows, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                               hipStream_t stream) {
     if (rows == 0) return launch_colreduce(dw, nullptr, nullptr, nullptr, 1, 0, cols, cols, dtype, stream);
     const GeomChoice gc = geometry_for(cols, dtype);
     RowPlan p;
@@ -617,7 +724,7 @@ int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, 
     const size_t need = (size_t)p.blocks * cols * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
-    st = dispatch<RmsBwd>(dtype, gc, p, dx, ws, g, x, w, rstd, rows, (int)cols, stream);
+    st = dispatch<RmsOn<Map>::template Bwd>(dtype, gc, p, dx, ws, g, x, w, rstd, map, (int)cols, stream);
     if (st != TT_NORM_OK) return st;
     st = check_launch("rmsnorm backward launch");
     if (st != TT_NORM_OK) return st;
@@ -625,41 +732,114 @@ int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, 
                             stream);
 }
 
-int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
-                           const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
-                           int dtype, hipStream_t stream) {
+int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
+                              const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
+                              size_t ws_bytes, hipStream_t stream) {
+    return rmsnorm_backward_on(dx, dw, g, x, w, rstd, DenseRows{rows}, rows, cols, dtype, ws, ws_bytes, stream);
+}
+
+int anywidth_rmsnorm_backward_strided(void *dx, void *dw, const void *g, const void *x, const void *w,
+                                      const float *rstd, const Strided3Rows &map, int64_t cols, int dtype,
+                                      void *ws, size_t ws_bytes, hipStream_t stream) {
+    return rmsnorm_backward_on(dx, dw, g, x, w, rstd, map, map.n0 * map.n1 * map.n2, cols, dtype, ws, ws_bytes,
+                               stream);
+}
+
+static SampleLayout layout_of(int64_t batch, int64_t rows_per_sample, bool seq_first) {
+    return seq_first ? SampleLayout{1, batch} : SampleLayout{rows_per_sample, 1};
+}
+
+bool anywidth_wide_forms_supported(int64_t cols, int dtype) {
+    return anywidth_supported(cols, dtype) && geometry_for(cols, dtype).chunks <= 6;
+}
+
+template <bool GATED>
+static int adaln_forward_any(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                             const void *shift, const AdalnExtra &ex, int64_t batch, int64_t rows_per_sample,
+                             int64_t cols, double eps, int dtype, bool seq_first, hipStream_t stream) {
     if (rows_per_sample == 0) return TT_NORM_OK;
     const GeomChoice gc = geometry_for(cols, dtype);
     RowPlan p;
     int st = plan_for(&p, batch, rows_per_sample, gc, false);
     if (st != TT_NORM_OK) return st;
-    st = dispatch<AdalnFwd>(dtype, gc, p, out, mean, rstd, x, scale, shift, rows_per_sample, (int)cols, eps, stream);
+    st = dispatch<AdalnOn<GATED, false>::template Fwd>(dtype, gc, p, out, mean, rstd, x, scale, shift, ex, rows_per_sample,
+                                                       layout_of(batch, rows_per_sample, seq_first), (int)cols, eps,
+                                                       stream);
     return st != TT_NORM_OK ? st : check_launch("adaln forward launch");
+}
+
+int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                           const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
+                           int dtype, hipStream_t stream, bool seq_first) {
+    return adaln_forward_any<false>(out, mean, rstd, x, scale, shift, AdalnExtra{nullptr, nullptr, nullptr, nullptr},
+                                    batch, rows_per_sample, cols, eps, dtype, seq_first, stream);
+}
+
+int anywidth_gated_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h, const void *attn,
+                                 const void *gate, const void *scale, const void *shift, int64_t batch,
+                                 int64_t rows_per_sample, int64_t cols, double eps, int dtype, hipStream_t stream) {
+    return adaln_forward_any<true>(out, mean, rstd, h, scale, shift, AdalnExtra{h2, nullptr, attn, gate}, batch,
+                                   rows_per_sample, cols, eps, dtype, false, stream);
 }
 
 size_t anywidth_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
     return backward_scratch(batch, rows_per_sample, cols, dtype, 2);
 }
 
-int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x,
-                            const void *scale, const float *mean, const float *rstd, int64_t batch,
-                            int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
-                            hipStream_t stream) {
+template <bool GATED, bool RES>
+static int adaln_backward_any(void *dx, void *dscale, void *dshift, void *dgate, const void *g, const void *x,
+                              const void *scale, const float *mean, const float *rstd, const AdalnExtra &ex,
+                              int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                              size_t ws_bytes, bool seq_first, hipStream_t stream) {
+    constexpr int NSETS = GATED ? 3 : 2;
     if (rows_per_sample == 0)
-        return launch_colreduce(dscale, dshift, nullptr, nullptr, batch, 0, cols, 2 * cols, dtype, stream);
+        return launch_colreduce(dscale, dshift, dgate, nullptr, batch, 0, cols, NSETS * cols, dtype, stream);
     const GeomChoice gc = geometry_for(cols, dtype);
     RowPlan p;
     int st = plan_for(&p, batch, rows_per_sample, gc, true);
     if (st != TT_NORM_OK) return st;
-    const size_t need = (size_t)p.blocks * 2 * cols * sizeof(float);
+    const size_t need = (size_t)p.blocks * NSETS * cols * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
-    st = dispatch<AdalnBwd>(dtype, gc, p, dx, ws, g, x, scale, mean, rstd, rows_per_sample, (int)cols, stream);
+    st = dispatch<AdalnOn<GATED, RES>::template Bwd>(dtype, gc, p, dx, ws, g, x, scale, mean, rstd, ex, rows_per_sample,
+                                                     layout_of(batch, rows_per_sample, seq_first), (int)cols, stream);
     if (st != TT_NORM_OK) return st;
     st = check_launch("adaln backward launch");
     if (st != TT_NORM_OK) return st;
-    return launch_colreduce(dscale, dshift, nullptr, (const float *)ws, batch, p.blocks_per_sample, cols, 2 * cols,
+    return launch_colreduce(dscale, dshift, dgate, (const float *)ws, batch, p.blocks_per_sample, cols, NSETS * cols,
                             dtype, stream);
+}
+
+int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x,
+                            const void *scale, const float *mean, const float *rstd, int64_t batch,
+                            int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                            hipStream_t stream, bool seq_first) {
+    return adaln_backward_any<false, false>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
+                                            AdalnExtra{nullptr, nullptr, nullptr, nullptr}, batch, rows_per_sample, cols,
+                                            dtype, ws, ws_bytes, seq_first, stream);
+}
+
+int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *g, const void *dres,
+                                     const void *x, const void *scale, const float *mean, const float *rstd,
+                                     int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                                     size_t ws_bytes, hipStream_t stream) {
+    return adaln_backward_any<false, true>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
+                                           AdalnExtra{nullptr, dres, nullptr, nullptr}, batch, rows_per_sample, cols, dtype,
+                                           ws, ws_bytes, false, stream);
+}
+
+size_t anywidth_gated_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
+    return backward_scratch(batch, rows_per_sample, cols, dtype, 3);
+}
+
+int anywidth_gated_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift, const void *g,
+                                  const void *dh2, const void *h2, const void *attn, const void *gate,
+                                  const void *scale, const float *mean, const float *rstd, int64_t batch,
+                                  int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                                  hipStream_t stream) {
+    return adaln_backward_any<true, false>(dh, dscale, dshift, dgate, g, h2, scale, mean, rstd,
+                                           AdalnExtra{dattn, dh2, attn, gate}, batch, rows_per_sample, cols, dtype, ws,
+                                           ws_bytes, false, stream);
 }
 
 }  // namespace ttn

@@ -43,10 +43,10 @@ void torch_launch_adaln_forward(torch::Tensor &output, torch::Tensor &x_norm, co
              "tt_adaln_forward_xnorm");
 }
 
-void torch_launch_adaln_forward_stats(torch::Tensor &output, const torch::Tensor &input,
-                                      const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
-                                      int64_t cols, double epsilon, torch::Tensor &mean,
-                                      torch::Tensor &inv_variance) {
+static void adaln_forward_stats_impl(torch::Tensor &output, const torch::Tensor &input,
+                                     const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                     int64_t cols, double epsilon, torch::Tensor &mean,
+                                     torch::Tensor &inv_variance, bool seq_first) {
     const auto dev = input.device();
     for (auto *t : {&output, &mean, &inv_variance}) check_dense_on(*t, dev, "output tensor");
     for (auto *t : {&input, &scale, &shift}) check_dense_on(*t, dev, "input tensor");
@@ -59,16 +59,38 @@ void torch_launch_adaln_forward_stats(torch::Tensor &output, const torch::Tensor
     check_elems(mean, rows, at::kFloat, "mean");
     check_elems(inv_variance, rows, at::kFloat, "inv_variance");
     c10::DeviceGuard guard(dev);
-    raise_on(tt_adaln_forward(output.data_ptr(), mean.data_ptr<float>(), inv_variance.data_ptr<float>(),
-                              input.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch, s.rows_per_sample,
-                              cols, epsilon, s.dt, current_stream(input)),
-             "tt_adaln_forward");
+    if (seq_first)
+        raise_on(tt_adaln_forward_seq_first(output.data_ptr(), mean.data_ptr<float>(), inv_variance.data_ptr<float>(),
+                                            input.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch,
+                                            s.rows_per_sample, cols, epsilon, s.dt, current_stream(input)),
+                 "tt_adaln_forward_seq_first");
+    else
+        raise_on(tt_adaln_forward(output.data_ptr(), mean.data_ptr<float>(), inv_variance.data_ptr<float>(),
+                                  input.data_ptr(), scale.data_ptr(), shift.data_ptr(), s.batch, s.rows_per_sample,
+                                  cols, epsilon, s.dt, current_stream(input)),
+                 "tt_adaln_forward");
+}
+
+void torch_launch_adaln_forward_stats(torch::Tensor &output, const torch::Tensor &input,
+                                      const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                      int64_t cols, double epsilon, torch::Tensor &mean,
+                                      torch::Tensor &inv_variance) {
+    adaln_forward_stats_impl(output, input, scale, shift, rows, cols, epsilon, mean, inv_variance, false);
+}
+
+// input is [rows / batch, batch, cols] (sequence first): sample b owns rows b, b + batch, ...
+void torch_launch_adaln_forward_stats_seq_first(torch::Tensor &output, const torch::Tensor &input,
+                                                const torch::Tensor &scale, const torch::Tensor &shift, int64_t rows,
+                                                int64_t cols, double epsilon, torch::Tensor &mean,
+                                                torch::Tensor &inv_variance) {
+    adaln_forward_stats_impl(output, input, scale, shift, rows, cols, epsilon, mean, inv_variance, true);
 }
 
 static void adaln_backward_impl(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
                                 const torch::Tensor &dout, const torch::Tensor &saved,
                                 const torch::Tensor &scale, const torch::Tensor *mean,
-                                const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+                                const torch::Tensor &inv_variance, int64_t rows, int64_t cols,
+                                bool seq_first = false) {
     const auto dev = dout.device();
     for (auto *t : {&dinp, &dscale, &dshift}) check_dense_on(*t, dev, "output tensor");
     for (auto *t : {&dout, &saved, &scale, &inv_variance}) check_dense_on(*t, dev, "input tensor");
@@ -89,7 +111,13 @@ static void adaln_backward_impl(torch::Tensor &dinp, torch::Tensor &dscale, torc
     const size_t need = tt_adaln_backward_workspace_bytes(s.batch, s.rows_per_sample, cols, s.dt);
     TORCH_CHECK(need > 0 || rows == 0, "unsupported AdaLN shape: cols=", cols);
     at::Tensor ws = scratch(need, dout);
-    if (mean)
+    if (mean && seq_first)
+        raise_on(tt_adaln_backward_seq_first(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(),
+                                             saved.data_ptr(), scale.data_ptr(), mean->data_ptr<float>(),
+                                             inv_variance.data_ptr<float>(), s.batch, s.rows_per_sample, cols, s.dt,
+                                             ws.data_ptr(), need, current_stream(dout)),
+                 "tt_adaln_backward_seq_first");
+    else if (mean)
         raise_on(tt_adaln_backward(dinp.data_ptr(), dscale.data_ptr(), dshift.data_ptr(), dout.data_ptr(),
                                    saved.data_ptr(), scale.data_ptr(), mean->data_ptr<float>(),
                                    inv_variance.data_ptr<float>(), s.batch, s.rows_per_sample, cols, s.dt,
@@ -117,6 +145,13 @@ void torch_launch_adaln_backward_x(torch::Tensor &dinp, torch::Tensor &dscale, t
                                    const torch::Tensor &scale, const torch::Tensor &mean,
                                    const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
     adaln_backward_impl(dinp, dscale, dshift, dout, input, scale, &mean, inv_variance, rows, cols);
+}
+
+void torch_launch_adaln_backward_x_seq_first(torch::Tensor &dinp, torch::Tensor &dscale, torch::Tensor &dshift,
+                                             const torch::Tensor &dout, const torch::Tensor &input,
+                                             const torch::Tensor &scale, const torch::Tensor &mean,
+                                             const torch::Tensor &inv_variance, int64_t rows, int64_t cols) {
+    adaln_backward_impl(dinp, dscale, dshift, dout, input, scale, &mean, inv_variance, rows, cols, true);
 }
 
 // Native backward for an input with another consumer: `dres` is the gradient the input receives from it,
@@ -225,6 +260,10 @@ PYBIND11_MODULE(fused_adaln, m) {
           "AdaLN forward kernel that saves mean and inv_variance instead of x_norm");
     m.def("torch_launch_adaln_backward_x", &torch_launch_adaln_backward_x,
           "AdaLN backward kernel (from the saved input and statistics)");
+    m.def("torch_launch_adaln_forward_stats_seq_first", &torch_launch_adaln_forward_stats_seq_first,
+          "AdaLN forward kernel on sequence-first rows [S, B, C]");
+    m.def("torch_launch_adaln_backward_x_seq_first", &torch_launch_adaln_backward_x_seq_first,
+          "AdaLN backward kernel on sequence-first rows [S, B, C]");
     m.def("supported", [](int64_t cols, const torch::Tensor &like) {
         return tt_norm_supported(cols, like.scalar_type() == at::kBFloat16 ? TT_NORM_BF16
                                        : like.scalar_type() == at::kFloat  ? TT_NORM_F32

@@ -346,6 +346,76 @@ __device__ __forceinline__ void row_pipeline(int64_t grp, int64_t groups, int64_
     }
 }
 
+// ---- where a wavefront's rows live ---------------------------------------------
+// A row map turns (wavefront group index, row within the wavefront) into the
+// row's logical number -- its index in the contiguous tensors (out, dout) and in
+// the per-row statistics -- and its element offsets in the tensors that may be
+// strided (x and, for backward, dx).
+struct RowAddr {
+    int64_t row;   // logical row number
+    int64_t xoff;  // element offset of the row in x
+    int64_t doff;  // element offset of the row in dx (backward only)
+    int64_t seq;   // index along the view's last leading dimension (the token of a [B, H, S, D] view)
+    bool ok;
+};
+
+// Row-major contiguous [rows, C].
+struct DenseRows {
+    int64_t rows;
+    template <int RPW>
+    __device__ __forceinline__ int64_t groups() const { return (rows + RPW - 1) / RPW; }
+    template <int RPW>
+    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub, int C) const {
+        RowAddr a;
+        a.row = grp * RPW + sub;
+        a.ok = a.row < rows;
+        a.xoff = a.doff = a.row * C;
+        a.seq = a.row;
+        return a;
+    }
+};
+
+// A 4-D view [n0, n1, n2, C] with contiguous last dimension and arbitrary other
+// strides (in elements); logical row number (i0*n1 + i1)*n2 + i2.  This is the
+// per-head QK-norm input: query.transpose(1, 2) is [B, H, S, D] with strides
+// (S*H*3D, 3D, H*3D, 1) inside the fused QKV projection output.
+// Traversal: a wavefront takes RPW consecutive i2 of one (i0, i1) -- so what it
+// writes to the contiguous side is one unbroken run -- and consecutive wavefronts
+// take consecutive i1 for the same i2 tile, so the workgroups running at the
+// same time read neighbouring pieces of the strided side.
+struct Strided3Rows {
+    int64_t n0, n1, n2;
+    int64_t xs0, xs1, xs2;
+    int64_t ds0, ds1, ds2;
+    template <int RPW>
+    __device__ __forceinline__ int64_t groups() const { return n0 * n1 * ((n2 + RPW - 1) / RPW); }
+    template <int RPW>
+    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub, int /*C*/) const {
+        const int64_t tiles2 = (n2 + RPW - 1) / RPW;
+        const int64_t i1 = grp % n1;
+        const int64_t q = grp / n1;
+        const int64_t i2 = (q % tiles2) * RPW + sub;
+        const int64_t i0 = q / tiles2;
+        RowAddr a;
+        a.ok = i2 < n2;
+        a.seq = i2;
+        a.row = (i0 * n1 + i1) * n2 + i2;
+        a.xoff = i0 * xs0 + i1 * xs1 + i2 * xs2;
+        a.doff = i0 * ds0 + i1 * ds1 + i2 * ds2;
+        return a;
+    }
+};
+
+// Where the rows of a sample live in the AdaLN tensors (x, out, dout, dx and the per-row statistics all
+// share it), in units of rows: row(b, r) = b * sample_stride + r * row_stride.
+//   sample-major [batch, rows_per_sample, C]: {rows_per_sample, 1}
+//   sequence-first [rows_per_sample, batch, C] (the layout of the blocks' callers, where the modulation row
+//   of sample b applies to rows b, b + batch, ...; teletron/models/dit/dit_layerspec.py:72-78): {1, batch}
+struct SampleLayout {
+    int64_t sample_stride, row_stride;
+    __device__ __forceinline__ int64_t row(int64_t b, int64_t r) const { return b * sample_stride + r * row_stride; }
+};
+
 // Adds this workgroup's per-lane column accumulators (acc[k][j] belongs to
 // column (k*LANES + l)*VEC + j) across the rows of each wavefront and across
 // wavefronts in fixed order, and writes one fp32 row of NSETS*C partial sums.

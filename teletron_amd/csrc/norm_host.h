@@ -78,13 +78,37 @@ size_t anywidth_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int
 int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
                               const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
                               size_t ws_bytes, hipStream_t stream);
+// The same over a strided 4-D view (see Strided3Rows): out / dout / rstd contiguous in logical row order.
+int anywidth_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void *w, const Strided3Rows &map,
+                                     int64_t cols, double eps, int dtype, hipStream_t stream);
+int anywidth_rmsnorm_backward_strided(void *dx, void *dw, const void *g, const void *x, const void *w,
+                                      const float *rstd, const Strided3Rows &map, int64_t cols, int dtype,
+                                      void *ws, size_t ws_bytes, hipStream_t stream);
+// seq_first: rows laid out [rows_per_sample, batch] (sample b owns rows b, b + batch, ...) instead of
+// [batch, rows_per_sample]; x, out, dout, dx and the statistics all share the layout.
 int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
                            const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
-                           int dtype, hipStream_t stream);
+                           int dtype, hipStream_t stream, bool seq_first = false);
 size_t anywidth_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype);
 int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x,
                             const void *scale, const float *mean, const float *rstd, int64_t batch,
                             int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
-                            hipStream_t stream);
+                            hipStream_t stream, bool seq_first = false);
+// The gated residual and residual forms, for rows of up to six 16-byte accesses per lane
+// (anywidth_wide_forms_supported): same argument meaning as the C-ABI entry points that forward to them.
+bool anywidth_wide_forms_supported(int64_t cols, int dtype);
+int anywidth_gated_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h, const void *attn,
+                                 const void *gate, const void *scale, const void *shift, int64_t batch,
+                                 int64_t rows_per_sample, int64_t cols, double eps, int dtype, hipStream_t stream);
+size_t anywidth_gated_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype);
+int anywidth_gated_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift, const void *g,
+                                  const void *dh2, const void *h2, const void *attn, const void *gate,
+                                  const void *scale, const float *mean, const float *rstd, int64_t batch,
+                                  int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                                  hipStream_t stream);
+int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *g, const void *dres,
+                                     const void *x, const void *scale, const float *mean, const float *rstd,
+                                     int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                                     size_t ws_bytes, hipStream_t stream);
 
 }  // namespace ttn

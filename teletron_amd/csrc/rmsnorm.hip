@@ -49,66 +49,6 @@
 
 namespace ttn {
 
-// ---- where a wavefront's rows live ---------------------------------------------
-// A row map turns (wavefront group index, row within the wavefront) into the
-// row's logical number -- its index in the contiguous tensors (out, dout) and in
-// the per-row statistics -- and its element offsets in the tensors that may be
-// strided (x and, for backward, dx).
-struct RowAddr {
-    int64_t row;   // logical row number
-    int64_t xoff;  // element offset of the row in x
-    int64_t doff;  // element offset of the row in dx (backward only)
-    int64_t seq;   // index along the view's last leading dimension (the token of a [B, H, S, D] view)
-    bool ok;
-};
-
-// Row-major contiguous [rows, C].
-struct DenseRows {
-    int64_t rows;
-    template <int RPW>
-    __device__ __forceinline__ int64_t groups() const { return (rows + RPW - 1) / RPW; }
-    template <int RPW, int C>
-    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub) const {
-        RowAddr a;
-        a.row = grp * RPW + sub;
-        a.ok = a.row < rows;
-        a.xoff = a.doff = a.row * C;
-        a.seq = a.row;
-        return a;
-    }
-};
-
-// A 4-D view [n0, n1, n2, C] with contiguous last dimension and arbitrary other
-// strides (in elements); logical row number (i0*n1 + i1)*n2 + i2.  This is the
-// per-head QK-norm input: query.transpose(1, 2) is [B, H, S, D] with strides
-// (S*H*3D, 3D, H*3D, 1) inside the fused QKV projection output.
-// Traversal: a wavefront takes RPW consecutive i2 of one (i0, i1) -- so what it
-// writes to the contiguous side is one unbroken run -- and consecutive wavefronts
-// take consecutive i1 for the same i2 tile, so the workgroups running at the
-// same time read neighbouring pieces of the strided side.
-struct Strided3Rows {
-    int64_t n0, n1, n2;
-    int64_t xs0, xs1, xs2;
-    int64_t ds0, ds1, ds2;
-    template <int RPW>
-    __device__ __forceinline__ int64_t groups() const { return n0 * n1 * ((n2 + RPW - 1) / RPW); }
-    template <int RPW, int C>
-    __device__ __forceinline__ RowAddr locate(int64_t grp, int sub) const {
-        const int64_t tiles2 = (n2 + RPW - 1) / RPW;
-        const int64_t i1 = grp % n1;
-        const int64_t q = grp / n1;
-        const int64_t i2 = (q % tiles2) * RPW + sub;
-        const int64_t i0 = q / tiles2;
-        RowAddr a;
-        a.ok = i2 < n2;
-        a.seq = i2;
-        a.row = (i0 * n1 + i1) * n2 + i2;
-        a.xoff = i0 * xs0 + i1 * xs1 + i2 * xs2;
-        a.doff = i0 * ds0 + i1 * ds1 + i2 * ds2;
-        return a;
-    }
-};
-
 // ---- rotary embedding behind the norm -----------------------------------------
 // The attention caller rotates the normalised query and key right after the per-head norm
 // (teletron/models/dit/dit_attention.py:266-273, :435-443) with the real-pair form of
@@ -187,7 +127,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
         keep_packed(wr);
-        const RowAddr at = map.template locate<RPW, C>(grp, sub);
+        const RowAddr at = map.template locate<RPW>(grp, sub, C);
         const int64_t row = at.row;
         const bool ok = at.ok;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(x + at.xoff) + l;
@@ -208,7 +148,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
         if (ok && l == 0) rstd[row] = r;
 
         // the wavefront's rows are consecutive in out: base = its first row
-        const int64_t row0 = map.template locate<RPW, C>(grp, 0).row;
+        const int64_t row0 = map.template locate<RPW>(grp, 0, C).row;
         const RowWriter<TTN_RMS_FWD_STORE> wo(out + row0 * C, (uint32_t)((sub * C) * sizeof(T)) + l * 16);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
@@ -294,10 +234,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         bool ok;
     };
     auto fetch = [&](RowRegs &b, int64_t grp) {
-        const RowAddr at = map.template locate<RPW, C>(grp, sub);
+        const RowAddr at = map.template locate<RPW>(grp, sub, C);
         b.ok = at.ok;
         b.seq = at.seq;
-        b.doff0 = map.template locate<RPW, C>(grp, 0).doff;
+        b.doff0 = map.template locate<RPW>(grp, 0, C).doff;
         b.dlane = (uint32_t)((at.doff - b.doff0) * (int64_t)sizeof(T)) + l * 16;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
@@ -572,10 +512,12 @@ int tt_rmsnorm_forward_strided(void *out, float *rstd, const void *x, const void
     int st = check_strided("tt_rmsnorm_forward_strided", n0, n1, n2, cols, dtype, xs, "x");
     if (st != TT_NORM_OK) return st;
     const int64_t rows = n0 * n1 * n2;
-    st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight}, true);
+    st = check_rms_args("tt_rmsnorm_forward_strided", rows, cols, dtype, {out, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!rstd && rows > 0) return fail(TT_NORM_EINVAL, "tt_rmsnorm_forward_strided: null rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, 0, 0, 0};
+    if (!tuned_shape(cols, dtype))
+        return anywidth_rmsnorm_forward_strided(out, rstd, x, weight, map, cols, eps, dtype, (hipStream_t)stream);
 #define CALL(T, C) return rmsnorm_forward_t<T, C>(out, rstd, x, weight, map, rows, eps, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
@@ -591,10 +533,13 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
     if (st == TT_NORM_OK) st = check_strided("tt_rmsnorm_backward_strided", n0, n1, n2, cols, dtype, ds, "dx");
     if (st != TT_NORM_OK) return st;
     const int64_t rows = n0 * n1 * n2;
-    st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight}, true);
+    st = check_rms_args("tt_rmsnorm_backward_strided", rows, cols, dtype, {dx, dout, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward_strided: null dweight/rstd");
     const Strided3Rows map{n0, n1, n2, xs0, xs1, xs2, dxs0, dxs1, dxs2};
+    if (!tuned_shape(cols, dtype))
+        return anywidth_rmsnorm_backward_strided(dx, dweight, dout, x, weight, rstd, map, cols, dtype, workspace,
+                                                 workspace_bytes, (hipStream_t)stream);
 #define CALL(T, C)                                                                                       \
     return rmsnorm_backward_t<T, C, false>(dx, dweight, dout, x, weight, rstd, map, rows, dtype, workspace, \
                                            workspace_bytes, (hipStream_t)stream)

@@ -47,7 +47,8 @@ except ImportError as exc:  # pragma: no cover - exercised only on an unbuilt tr
     log.warning("fused_adaln / fused_rmsnorm extensions not importable (%s); "
                 "build them with `python -m teletron_amd.build`.", exc)
 
-TUNED_COLS = (128, 3072)  # the reference's two shapes; strided views and the gated op need these
+TUNED_COLS = (128, 3072)  # the reference's two shapes (the tuned kernels)
+_WIDE_FORM_PIECES = 384   # gated / residual forms: 3072 columns, or any row of up to this many 16-byte pieces
 _ELEM_BYTES = {torch.bfloat16: 2, torch.float16: 2, torch.float32: 4}
 _MAX_PIECES = 1024  # 16-byte pieces per row the kernels are built for
 
@@ -60,6 +61,11 @@ def cols_supported(cols: int, dtype: torch.dtype) -> bool:
         return False
     vec = 16 // size
     return cols % vec == 0 and cols // vec <= _MAX_PIECES
+
+
+def wide_forms_supported(cols: int, dtype: torch.dtype) -> bool:
+    """Whether the gated residual + AdaLN and the stream-keeping AdaLN take rows of `cols` elements."""
+    return cols_supported(cols, dtype) and (cols == 3072 or cols * _ELEM_BYTES[dtype] // 16 <= _WIDE_FORM_PIECES)
 
 
 def _unsupported(cols: int, dtype: torch.dtype) -> str:
@@ -110,11 +116,16 @@ class AdaLNModelFunction(Function):
     apply(x, scale, shift, epsilon, cols) -> out, with gradients for x, scale
     and shift (dit_fusedlayers.py:66,108).  x is [..., cols]; scale and shift are
     [cols] or [B, cols] with B == x.shape[0] (one modulation row per sample).
+    A sixth argument True says x is sequence-first, [S, B, cols] with B == x.shape[1]
+    (the layout the output norm sees, dit_layerspec.py:72-78): it is normalised in place,
+    without regrouping the rows by sample.
     """
 
     @staticmethod
-    def forward(ctx, x, scale, shift, epsilon, cols):
+    def forward(ctx, x, scale, shift, epsilon, cols, *seq_first):
         ext = _require_extension(fused_adaln, "fused_adaln")
+        ctx.n_extra = len(seq_first)
+        seq_first = bool(seq_first[0]) if seq_first else False
         _require_gpu(x, "AdaLNModelFunction")
         x = _aligned_contiguous(x)
         scale_c = scale.contiguous()
@@ -127,7 +138,10 @@ class AdaLNModelFunction(Function):
         if scale_c.numel() % cols != 0 or shift_c.numel() != scale_c.numel():
             raise ValueError(f"scale/shift sizes {scale_c.numel()}/{shift_c.numel()} do not match cols {cols}")
         batch = scale_c.numel() // cols
-        if batch > 1 and (x.dim() < 2 or x.shape[0] != batch):
+        if seq_first:
+            if x.dim() != 3 or x.shape[1] != batch:
+                raise ValueError(f"sequence-first input must be [S, {batch}, {cols}], got {tuple(x.shape)}")
+        elif batch > 1 and (x.dim() < 2 or x.shape[0] != batch):
             raise ValueError(f"{batch} modulation rows need x.shape[0] == {batch}, got {tuple(x.shape)}")
         if scale_c.dtype != x.dtype or shift_c.dtype != x.dtype:
             scale_c, shift_c = scale_c.to(x.dtype), shift_c.to(x.dtype)
@@ -135,9 +149,10 @@ class AdaLNModelFunction(Function):
         out = torch.empty_like(x)
         mean = torch.empty(rows, device=x.device, dtype=torch.float32)
         invvar = torch.empty(rows, device=x.device, dtype=torch.float32)
-        ext.torch_launch_adaln_forward_stats(out, x, scale_c, shift_c, rows, cols, float(epsilon), mean, invvar)
+        launch = ext.torch_launch_adaln_forward_stats_seq_first if seq_first else ext.torch_launch_adaln_forward_stats
+        launch(out, x, scale_c, shift_c, rows, cols, float(epsilon), mean, invvar)
         ctx.save_for_backward(x, scale_c, mean, invvar)
-        ctx.rows, ctx.cols = rows, cols
+        ctx.rows, ctx.cols, ctx.seq_first = rows, cols, seq_first
         ctx.mod_shape, ctx.mod_dtype = scale.shape, scale.dtype
         return out
 
@@ -150,11 +165,12 @@ class AdaLNModelFunction(Function):
         grad_input = torch.empty_like(x)
         grad_scale = torch.empty_like(scale_c)
         grad_shift = torch.empty_like(scale_c)
-        fused_adaln.torch_launch_adaln_backward_x(grad_input, grad_scale, grad_shift, grad_output, x, scale_c,
-                                                  mean, invvar, ctx.rows, ctx.cols)
+        launch = (fused_adaln.torch_launch_adaln_backward_x_seq_first if ctx.seq_first
+                  else fused_adaln.torch_launch_adaln_backward_x)
+        launch(grad_input, grad_scale, grad_shift, grad_output, x, scale_c, mean, invvar, ctx.rows, ctx.cols)
         grad_scale = grad_scale.reshape(ctx.mod_shape).to(ctx.mod_dtype)
         grad_shift = grad_shift.reshape(ctx.mod_shape).to(ctx.mod_dtype)
-        return grad_input, grad_scale, grad_shift, None, None
+        return (grad_input, grad_scale, grad_shift, None, None) + (None,) * ctx.n_extra
 
 
 class AdaLNResidualFunction(Function):
@@ -162,15 +178,17 @@ class AdaLNResidualFunction(Function):
     itself, handed back as an output for the caller to continue the residual stream with
     (dit_layerspec.py:126-131 then :152).  Routing the stream through the Function lets backward add the
     gradient it collected downstream to the norm's dx inside the kernel, in place of the separate
-    accumulation pass autograd runs when a tensor has two consumers.  3072 columns."""
+    accumulation pass autograd runs when a tensor has two consumers.  3072 columns, or any supported row of up
+    to 3072 two-byte / 1536 four-byte columns."""
 
     @staticmethod
     def forward(ctx, x, scale, shift, epsilon):
         ext = _require_extension(fused_adaln, "fused_adaln")
         _require_gpu(x, "AdaLNResidualFunction")
         cols = x.shape[-1]
-        if cols != 3072 or x.dtype not in _ELEM_BYTES:
-            raise ValueError(f"AdaLNResidualFunction needs 3072 columns in bfloat16/float16/float32, got {cols}, {x.dtype}")
+        if x.dtype not in _ELEM_BYTES or not wide_forms_supported(cols, x.dtype):
+            raise ValueError(f"AdaLNResidualFunction: {_unsupported(cols, x.dtype)}; rows of at most 3072 two-byte / "
+                             "1536 four-byte columns, or 3072 columns")
         x_c = _aligned_contiguous(x)
         scale_c, shift_c = scale.contiguous().to(x.dtype), shift.contiguous().to(x.dtype)
         if scale_c.numel() % cols or shift_c.numel() != scale_c.numel():
@@ -230,12 +248,16 @@ class AdaLNCustom(nn.Module):
         return AdaLNModelFunction.apply(x, scale, shift, self.eps, cols)
 
 
-def modulated_layer_norm(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6):
+def modulated_layer_norm(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6,
+                         seq_first: bool = False):
     """LayerNorm(x) * (1 + scale[:, None]) + shift[:, None] through the fused kernel.
 
     The same math as the adaLN-Zero input norm; also what the reference leaves
     un-fused after attention (`norm2` + modulate, dit_layerspec.py:158-167) and
-    in the output head (AdaLNContinuous, dit_layerspec.py:55-78)."""
+    in the output head (AdaLNContinuous, dit_layerspec.py:55-78).  seq_first: x is [S, B, C]
+    and the result is LayerNorm(x) * (1 + scale) + shift broadcast over S, in place."""
+    if seq_first:
+        return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1], True)
     return AdaLNModelFunction.apply(x, scale, shift, eps, x.shape[-1])
 
 
@@ -247,13 +269,16 @@ class GatedResidualAdaLNFunction(Function):
     (dit_layerspec.py:152-167, :351-352), which the reference runs as separate
     elementwise kernels around the norm.  h, attn [B, S, C]; gate, scale, shift [B, C].
     h2 is the new residual stream; its gradient from later uses is folded into the
-    same backward pass.  C must be 3072."""
+    same backward pass.  C: 3072, or any supported row of up to 3072 two-byte / 1536 four-byte columns."""
 
     @staticmethod
     def forward(ctx, h, attn, gate, scale, shift, epsilon):
         ext = _require_extension(fused_adaln, "fused_adaln")
         _require_gpu(h, "GatedResidualAdaLNFunction")
         cols = h.shape[-1]
+        if h.dtype not in _ELEM_BYTES or not wide_forms_supported(cols, h.dtype):
+            raise ValueError(f"GatedResidualAdaLNFunction: {_unsupported(cols, h.dtype)}; rows of at most 3072 two-byte "
+                             "/ 1536 four-byte columns, or 3072 columns")
         if attn.shape != h.shape:
             raise ValueError(f"attn {tuple(attn.shape)} must have the shape of h {tuple(h.shape)}")
         mods = [t.contiguous().to(h.dtype) for t in (gate, scale, shift)]
@@ -436,8 +461,7 @@ class RMSNormModelFunction(Function):
             raise ValueError(_unsupported(cols, x.dtype))
         if weight.numel() != cols:
             raise ValueError(f"weight has {weight.numel()} elements, expected cols {cols}")
-        tuned = cols in TUNED_COLS and x.dtype in _ELEM_BYTES
-        strided = tuned and x.shape[-1] == cols and _strided_rows_ok(x)
+        strided = x.shape[-1] == cols and _strided_rows_ok(x)
         if not strided:
             x = _aligned_contiguous(x)
         w = weight.contiguous()
@@ -503,7 +527,7 @@ class QKVSplitNormFunction(Function):
     Backward writes the gradients of q and k from the kernels directly into their slices of one
     [B, S, H, 3*D] gradient tensor and copies the gradient of v into its slice, so the concatenation
     that torch.split's backward would run over three separate gradients never happens.
-    D must be 128 or 3072."""
+    D: any supported row (128 runs the tuned kernels; the rotary form needs 128)."""
 
     @staticmethod
     def forward(ctx, mixed_qkv, weight_q, weight_k, epsilon, *rotary):
@@ -519,9 +543,8 @@ class QKVSplitNormFunction(Function):
         if mixed_qkv.dim() != 4 or mixed_qkv.shape[-1] % 3:
             raise ValueError(f"mixed_qkv must be [B, S, H, 3*D], got {tuple(mixed_qkv.shape)}")
         cols = mixed_qkv.shape[-1] // 3
-        if cols not in TUNED_COLS or mixed_qkv.dtype not in _ELEM_BYTES:
-            raise ValueError(f"QKVSplitNormFunction needs D in {TUNED_COLS} and bfloat16/float16/float32, got D={cols}, "
-                             f"{mixed_qkv.dtype}")
+        if mixed_qkv.dtype not in _ELEM_BYTES or not cols_supported(cols, mixed_qkv.dtype):
+            raise ValueError(f"QKVSplitNormFunction: {_unsupported(cols, mixed_qkv.dtype)}")
         tables = None
         if rotary:
             if cols != 128:
@@ -602,7 +625,7 @@ def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSN
     Fused when FUSED_KERNELS is on and the head dimension is one the tuned kernels take (128 for the
     rotary form); the reference's own sequence of operations otherwise."""
     D = mixed_qkv.shape[-1] // 3
-    fusable = (fused_kernels_requested() and D in TUNED_COLS and mixed_qkv.dtype in _ELEM_BYTES
+    fusable = (fused_kernels_requested() and mixed_qkv.dtype in _ELEM_BYTES and cols_supported(D, mixed_qkv.dtype)
                and q_norm.eps == k_norm.eps)
     if fusable and rotary is None:
         return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
@@ -656,8 +679,8 @@ class AdaLNContinuous(nn.Module):
         scale, shift = torch.chunk(emb, 2, dim=1)
         if not self.fused_kernels:
             return self.norm(x) * (1 + scale) + shift
-        if x.dim() == 3:    # [S, B, C]: the kernel wants a sample's rows together
-            return modulated_layer_norm(x.transpose(0, 1), scale, shift, eps=1e-6).transpose(0, 1)
+        if x.dim() == 3:    # [S, B, C]: normalised where it lies, sample b owning rows b, b + B, ...
+            return modulated_layer_norm(x, scale, shift, eps=1e-6, seq_first=True)
         if x.dim() == 2:    # [B, C]: one row per sample
             return modulated_layer_norm(x.unsqueeze(1), scale, shift, eps=1e-6).squeeze(1)
         raise ValueError(f"AdaLNContinuous expects x of [S, B, C] or [B, C], got {tuple(x.shape)}")

@@ -124,7 +124,7 @@ def test_unsupported_widths_and_entry_points(capi, gpu_device):
         with pytest.raises(capi.NormError) as e:
             capi.rmsnorm_forward(mk(4, cols, dt=dt), mk(cols, dt=dt), EPS)
         assert e.value.status == 2
-    # reference-contract and strided entry points exist for the tuned shapes only
+    # reference-contract entry points exist for the tuned shapes only
     with pytest.raises(capi.NormError) as e:
         capi.rmsnorm_backward(mk(4, 256), mk(4, 256), mk(256), torch.zeros(4, device=gpu_device), from_out=True)
     assert e.value.status == 2
@@ -235,3 +235,149 @@ def test_fp16_through_the_tuned_only_entry_points(capi, gpu_device):
     dx, _, _ = capi.adaln_backward(gr, x, dev_(sc), mean, rstd)
     dxr, _, _ = capi.adaln_backward_residual(gr, other, x, dev_(sc), mean, rstd)
     assert torch.equal(dxr, dx + other)
+
+
+# ------------------------- the call-site forms at other widths (strided, gated, residual, sequence-first)
+
+@pytest.mark.parametrize("D,dtype,B,S,H", [(64, BF, 2, 203, 5), (256, HF, 1, 77, 3), (96, F32, 1, 130, 2), (40, BF, 1, 9, 1)])
+def test_strided_qk_norm_at_other_head_dims(capi, gpu_device, D, dtype, B, S, H):
+    """The transposed [B, H, S, D] views into a fused [B, S, H, 3D] projection, read in place, for head
+    dimensions the tuned kernels are not built for: equal to the dense kernels on a contiguous copy bit for
+    bit, and to eager within the bars."""
+    gen = torch.Generator().manual_seed(D)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).to(dtype)
+    w = (1 + 0.02 * torch.randn(D, generator=gen)).to(dtype)
+    grad = torch.randn(B, H, S, D, generator=gen).to(dtype)
+    mixed_g, w_g, grad_g = mixed.to(gpu_device), w.to(gpu_device), grad.to(gpu_device)
+    for i in range(2):
+        x_cpu = mixed[..., i * D:(i + 1) * D].transpose(1, 2)
+        x_g = mixed_g[..., i * D:(i + 1) * D].transpose(1, 2)
+        assert not x_g.is_contiguous()
+        want_out, want_dx, want_dw = O.eager_rmsnorm_fwd_bwd(x_cpu, w, grad)
+        out, rstd = capi.rmsnorm_forward_strided(x_g, w_g, EPS)
+        dx, dw = capi.rmsnorm_backward_strided(grad_g, x_g, w_g, rstd)
+        out_d, rstd_d = capi.rmsnorm_forward(x_g.contiguous(), w_g, EPS)
+        dx_d, dw_d = capi.rmsnorm_backward(grad_g, x_g.contiguous(), w_g, rstd_d)
+        assert torch.equal(out, out_d) and torch.equal(rstd, rstd_d)
+        assert torch.equal(dx.contiguous(), dx_d)
+        # (the strided traversal hands rows to wavefronts in another order, so dweight's fp32 partial sums
+        # associate differently: equal after rounding to a 16-bit type, a few fp32 ulps apart otherwise)
+        torch.testing.assert_close(dw.float(), dw_d.float(), rtol=1e-5, atol=1e-4)
+        if dtype == F32:
+            torch.testing.assert_close(out.cpu(), want_out, rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(dx.cpu(), want_dx, rtol=1e-4, atol=1e-5)
+        else:
+            fwd_16bit_ok(out, want_out, O.rmsnorm_excuse(want_out), "out")
+            grad_ok(dx, want_dx, "dx")
+            grad_ok(dw, want_dw, "dweight")
+    # dx written through strides into a slice of one gradient tensor (what QKVSplitNormFunction does)
+    d_mixed = torch.zeros_like(mixed_g)
+    x_g = mixed_g[..., :D].transpose(1, 2)
+    out, rstd = capi.rmsnorm_forward_strided(x_g, w_g, EPS)
+    dx, _ = capi.rmsnorm_backward_strided(grad_g, x_g, w_g, rstd)
+    capi.rmsnorm_backward_strided(grad_g, x_g, w_g, rstd, dx=d_mixed[..., :D].transpose(1, 2))
+    assert torch.equal(d_mixed[..., :D].transpose(1, 2), dx) and not d_mixed[..., D:].any()
+
+
+@pytest.mark.parametrize("C,dtype,B,S,with_h2", [(1536, BF, 2, 515, True), (1024, HF, 3, 130, False), (512, F32, 2, 77, True),
+                                                 (2048, BF, 1, 300, True), (64, BF, 2, 1001, True), (1536, F32, 1, 65, False)])
+def test_gated_residual_adaln_at_other_widths(capi, gpu_device, C, dtype, B, S, with_h2):
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(B, S, C, dtype, seed=C + S, with_grad_h2=with_h2)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    to = lambda t: None if t is None else t.to(gpu_device)
+    H, A, Q, SC, SH, GO, G2 = (to(t) for t in (h, a, q, sc, sh, go, g2))
+    h2, out, mean, rstd = capi.gated_residual_adaln_forward(H, A, Q, SC, SH, EPS)
+    dh, da, dq, dsc, dsh = capi.gated_residual_adaln_backward(GO, G2, h2, A, Q, SC, mean, rstd)
+    # bit-identical to its parts run one after the other: elementwise update, plain AdaLN, plain backward + add
+    h2_parts = H + A * Q[:, None]
+    assert torch.equal(h2, h2_parts)
+    out_p, mean_p, rstd_p = capi.adaln_forward(h2_parts, SC, SH, EPS)
+    assert torch.equal(out, out_p) and torch.equal(mean, mean_p) and torch.equal(rstd, rstd_p)
+    dxn, dsc_p, dsh_p = capi.adaln_backward(GO, h2_parts, SC, mean_p, rstd_p)
+    dh_parts = dxn + G2 if with_h2 else dxn
+    assert torch.equal(dh, dh_parts) and torch.equal(da, dh_parts * Q[:, None])
+    assert torch.equal(dsc, dsc_p) and torch.equal(dsh, dsh_p)
+    if dtype == F32:
+        torch.testing.assert_close(out.cpu(), want[1], rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(dh.cpu(), want[2], rtol=1e-3, atol=1e-4)
+        l1 = (want[2].abs() * a.abs()).sum(1)
+        assert ((dq.cpu() - want[4]).abs() <= 1e-4 * l1 + 1e-5).all()
+    else:
+        assert torch.equal(h2.cpu(), want[0])
+        fwd_16bit_ok(out, want[1], O.adaln_excuse(want[0], sc, sh, want[1]), "out")
+        terms = O.adaln_dx_terms(want[0], sc, go) + (g2.float().abs() if with_h2 else 0)
+        assert O.frac_outside(dh.cpu(), want[2], 1e-2, 1e-3, magnitude=terms) <= 1e-4
+        assert O.colsum_outside(dq.cpu(), want[4], terms * a.float(), dim=1) == 0
+        colsum_ok(dsc, want[5], go.float() * 3, 1, "dscale")
+        colsum_ok(dsh, want[6], go.float(), 1, "dshift")
+
+
+@pytest.mark.parametrize("C,dtype", [(1536, BF), (1024, HF), (768, F32), (128, BF)])
+def test_adaln_backward_residual_at_other_widths(capi, gpu_device, C, dtype):
+    d = O.make_adaln_inputs(2, 301, C, dtype, seed=C)
+    other = O.make_adaln_inputs(2, 301, C, dtype, seed=C + 1)["grad"]
+    g = {k: v.to(gpu_device) for k, v in d.items()}
+    _, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    dx, ds, dh = capi.adaln_backward(g["grad"], g["x"], g["scale"], mean, rstd)
+    dxr, dsr, dhr = capi.adaln_backward_residual(g["grad"], other.to(gpu_device), g["x"], g["scale"], mean, rstd)
+    assert torch.equal(dxr, dx + other.to(gpu_device)) and torch.equal(dsr, ds) and torch.equal(dhr, dh)
+
+
+@pytest.mark.parametrize("C,dtype,B,S", [(3072, BF, 3, 129), (3072, F32, 2, 33), (1536, HF, 4, 65), (128, BF, 3, 1001),
+                                         (64, BF, 5, 77), (3072, BF, 1, 100), (4096, BF, 2, 40)])
+def test_adaln_on_sequence_first_rows(capi, gpu_device, C, dtype, B, S):
+    """x [S, B, C] with one modulation row per sample (the output norm's layout, dit_layerspec.py:72-78),
+    normalised where it lies: bit-identical to the sample-major call on the regrouped rows, statistics
+    included (they are indexed by the same row numbers as x)."""
+    d = O.make_adaln_inputs(B, S, C, dtype, seed=7 * C + B)
+    g = {k: v.to(gpu_device) for k, v in d.items()}
+    x_sf, grad_sf = g["x"].transpose(0, 1).contiguous(), g["grad"].transpose(0, 1).contiguous()   # [S, B, C]
+    out, mean, rstd = capi.adaln_forward(g["x"], g["scale"], g["shift"], EPS)
+    dx, ds, dh = capi.adaln_backward(g["grad"], g["x"], g["scale"], mean, rstd)
+    out_sf, mean_sf, rstd_sf = capi.adaln_forward(x_sf, g["scale"], g["shift"], EPS, seq_first=True)
+    dx_sf, ds_sf, dh_sf = capi.adaln_backward(grad_sf, x_sf, g["scale"], mean_sf, rstd_sf, seq_first=True)
+    assert torch.equal(out_sf.transpose(0, 1), out) and torch.equal(dx_sf.transpose(0, 1), dx)
+    assert torch.equal(mean_sf.reshape(S, B).t(), mean.reshape(B, S))
+    assert torch.equal(rstd_sf.reshape(S, B).t(), rstd.reshape(B, S))
+    assert torch.equal(ds_sf, ds) and torch.equal(dh_sf, dh)
+    # and the eager formula as the caller writes it: norm(x) * (1 + scale) + shift broadcast over S
+    if dtype != F32:
+        want = torch.nn.functional.layer_norm(d["x"].transpose(0, 1), (C,), None, None, EPS) * (1 + d["scale"]) + d["shift"]
+        assert O.frac_outside(out_sf.cpu(), want, 1e-2, 1e-2) <= 1e-4
+
+
+def test_functions_take_the_wide_forms_at_other_widths(gpu_device):
+    """The autograd Functions at hidden 1536: gated residual + AdaLN and the stream-keeping AdaLN, and
+    QKVSplitNormFunction at head dimension 64."""
+    from teletron_amd import fusedlayers as FL
+    h, a, q, sc, sh, go, g2 = O.make_gated_inputs(2, 130, 1536, BF, seed=5)
+    want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
+    leaves = [t.to(gpu_device).requires_grad_(True) for t in (h, a, q, sc, sh)]
+    h2, out = FL.gated_residual_layer_norm(*leaves, eps=EPS)
+    torch.autograd.backward([out, h2], [go.to(gpu_device), g2.to(gpu_device)])
+    assert torch.equal(h2.detach().cpu(), want[0])
+    fwd_16bit_ok(out.detach(), want[1], O.adaln_excuse(want[0], sc, sh, want[1]), "out")
+    grad_ok(leaves[3].grad, want[5], "dscale")
+    grad_ok(leaves[4].grad, want[6], "dshift")
+    x = h.to(gpu_device).requires_grad_(True)
+    same, out2 = FL.modulated_layer_norm_keeping_stream(x, sc.to(gpu_device), sh.to(gpu_device), EPS)
+    torch.autograd.backward([out2, same * 1.0], [go.to(gpu_device), g2.to(gpu_device)])
+    assert x.grad is not None and x.grad.shape == h.shape
+    with pytest.raises(ValueError, match="unsupported cols|rows of at most"):
+        FL.gated_residual_layer_norm(torch.zeros(1, 4, 4096, dtype=BF, device=gpu_device),
+                                     torch.zeros(1, 4, 4096, dtype=BF, device=gpu_device),
+                                     *(torch.zeros(1, 4096, dtype=BF, device=gpu_device) for _ in range(3)), eps=EPS)
+    B, S, H, D = 1, 101, 4, 64
+    gen = torch.Generator().manual_seed(64)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()
+    wq, wk = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16(), (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    gq, gk, gv = (torch.randn(B, H, S, D, generator=gen).bfloat16() for _ in range(3))
+    m_c = mixed.clone().requires_grad_(True)
+    q_c, k_c, v_c = torch.split(m_c, [D, D, D], dim=3)
+    q_c, k_c = O.eager_rmsnorm(q_c.transpose(1, 2), wq), O.eager_rmsnorm(k_c.transpose(1, 2), wk)
+    torch.autograd.backward([q_c, k_c, v_c.transpose(1, 2)], [gq, gk, gv])
+    m_g = mixed.to(gpu_device).requires_grad_(True)
+    q_g, k_g, v_g = FL.QKVSplitNormFunction.apply(m_g, wq.to(gpu_device), wk.to(gpu_device), EPS)
+    fwd_16bit_ok(q_g.detach(), q_c.detach(), O.rmsnorm_excuse(q_c.detach()), "q")
+    torch.autograd.backward([q_g, k_g, v_g], [gq.to(gpu_device), gk.to(gpu_device), gv.to(gpu_device)])
+    grad_ok(m_g.grad, m_c.grad, "d mixed")
