@@ -99,34 +99,36 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     const int64_t b = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
 
-    // This sample's modulation row, staged once per workgroup through LDS: each thread
-    // forms t = rnd(1 + scale) for its share of the 16-byte pieces, then every lane picks up
-    // the pieces of its own columns.  (One-shot wavefronts would otherwise each repeat the
-    // whole row: 12 loads and ~120 VALU instructions per 6 KiB of useful traffic.)
+    // This sample's modulation row, staged once per workgroup through LDS AS FP32: each thread forms
+    // t = rnd(1 + scale) for its share of the 16-byte pieces and stores t and shift unpacked, four
+    // floats per 16-byte slot in VEC/4 planes (plane p of piece i = elements 4p..4p+3, so a wavefront's
+    // 16-byte reads of one plane are contiguous).  The last pass then takes its parameters with LDS
+    // reads instead of unpacking them in the ALU: at 3072 two-byte columns that is 96 of ~800 VALU
+    // instructions per row, and this kernel is the one closest to being ALU-bound when the part
+    // runs at reduced clocks.  (One-shot wavefronts reading the row themselves would each repeat 12
+    // loads and ~120 VALU instructions per 6 KiB of useful traffic.)
     constexpr int kPieces = C / VEC;  // 16-byte pieces per parameter row
-    __shared__ u32x4 lds_t[kPieces], lds_h[kPieces], lds_g[GATED ? kPieces : 1];
+    constexpr int kPlanes = VEC / 4;
+    __shared__ u32x4 lds_t[kPlanes][kPieces], lds_h[kPlanes][kPieces], lds_g[GATED ? kPieces : 1];
     for (int i = threadIdx.x; i < kPieces; i += kRowThreads) {
-        float v[VEC];
+        float v[VEC], h[VEC];
         E::unpack(load16(reinterpret_cast<const u32x4 *>(scale + b * C) + i), v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
-        lds_t[i] = E::pack(v);
-        lds_h[i] = load16(reinterpret_cast<const u32x4 *>(shift + b * C) + i);
+        E::round(v);  // t = 1 + scale in the element type
+        E::unpack(load16(reinterpret_cast<const u32x4 *>(shift + b * C) + i), h);
+#pragma unroll
+        for (int p = 0; p < kPlanes; ++p) {
+            lds_t[p][i] = u32x4{as_u32(v[4 * p]), as_u32(v[4 * p + 1]), as_u32(v[4 * p + 2]), as_u32(v[4 * p + 3])};
+            lds_h[p][i] = u32x4{as_u32(h[4 * p]), as_u32(h[4 * p + 1]), as_u32(h[4 * p + 2]), as_u32(h[4 * p + 3])};
+        }
         if constexpr (GATED) lds_g[i] = load16(reinterpret_cast<const u32x4 *>(gate + b * C) + i);
     }
     __syncthreads();
-    u32x4 tr[CHUNKS], hr[CHUNKS];
-#pragma unroll
-    for (int k = 0; k < CHUNKS; ++k) {
-        tr[k] = lds_t[k * LANES + l];
-        hr[k] = lds_h[k * LANES + l];
-    }
 
     const int64_t groups = (rows_per_sample + RPW - 1) / RPW;
     const int64_t stride = (int64_t)blocks_per_sample * kRowWaves;
     for (int64_t grp = (int64_t)slot * kRowWaves + wave; grp < groups; grp += stride) {
-        keep_packed(tr);
-        keep_packed(hr);
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         const bool ok = rs < rows_per_sample;
         const int64_t row = lay.row(b, rs);
@@ -196,9 +198,18 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
             float v[VEC], tv[VEC], hv[VEC];
+            // keeps the LDS reads of later accesses from being hoisted up here, where they would all be live at once
+            if constexpr (CHUNKS > 1) __builtin_amdgcn_sched_barrier(0);
             E::unpack(xr[k], v);
-            E::unpack(tr[k], tv);
-            E::unpack(hr[k], hv);
+#pragma unroll
+            for (int p = 0; p < kPlanes; ++p) {
+                const u32x4 tq = lds_t[p][k * LANES + l], hq = lds_h[p][k * LANES + l];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    tv[4 * p + j] = as_f32(tq[j]);
+                    hv[4 * p + j] = as_f32(hq[j]);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] = centred<T>(v[j], mu, r, nmr);
             if constexpr (WRITE_XNORM) {
@@ -329,8 +340,10 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
             for (int k = 0; k < CHUNKS; ++k)
                 b.e[k] = (b.ok && e != nullptr) ? load16_stream(pe + k * LANES) : u32x4{0, 0, 0, 0};
         }
-        b.r = b.ok ? rstd[b.row] : 0.0f;
-        b.mu = (!FROM_XNORM && b.ok) ? mean[b.row] : 0.0f;
+        // one row per wavefront: its statistics come through the scalar cache
+        const int64_t srow = LANES == kWaveSize ? wave_uniform(b.row) : b.row;
+        b.r = b.ok ? rstd[srow] : 0.0f;
+        b.mu = (!FROM_XNORM && b.ok) ? mean[srow] : 0.0f;
     };
     auto process = [&](const RowRegs &b, auto &&between_passes) {
         const float r = b.r, mu = b.mu;

@@ -297,6 +297,14 @@ __device__ __forceinline__ float fold_rows_of_wave(float v) {
     return v;
 }
 
+// A 64-bit value every lane of the wavefront holds alike, moved to scalar registers: indexing a per-row
+// array with it is then a scalar load instead of a vector load that queues behind the row's own loads.
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 __device__ __forceinline__ int wave_id_in_block() {
     return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }
