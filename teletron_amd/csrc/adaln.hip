@@ -48,11 +48,14 @@
 // Dynamic LDS requested by the forward launch (0: none).  Only a throttle on how many
 // one-shot workgroups a compute unit holds at once; the kernel does not touch it.
 // AdaLN forward spends longer in the ALU per row than RMSNorm forward and wants all the
-// wavefronts its registers allow (16 per compute unit), so no throttle for 2-byte rows.  4-byte
-// rows carry twice the bytes per wavefront: 40 KiB on top of the 24 KiB of staged modulation rows
-// leaves two workgroups per compute unit (232 vs 244 us at 59 400 rows).
+// wavefronts its registers and its staged parameters allow (six workgroups per compute unit for
+// 2-byte rows: 236 us at 118 800 rows against 238 with four and 280 with three).  The gated form
+// moves twice the bytes per row (2 reads + 2 writes) and streams best with three workgroups per
+// compute unit (12 KiB on top of its 30 KiB: 482 vs 509 us between backward launches).  4-byte rows
+// carry twice the bytes per wavefront: 40 KiB on top of the staged modulation rows leaves two
+// workgroups per compute unit (232 vs 244 us at 59 400 rows).
 #ifndef TTN_ADALN_FWD_DYN_LDS
-#define TTN_ADALN_FWD_DYN_LDS (C >= 1024 && sizeof(T) == 4 ? 40960 : 0)
+#define TTN_ADALN_FWD_DYN_LDS (C >= 1024 ? (sizeof(T) == 4 ? 40960 : (GATED ? 12288 : 0)) : 0)
 #endif
 // Backward row fetch: all of g's accesses, then all of x's (two contiguous 6 KiB runs per
 // wavefront at 3072 columns) rather than alternating 1 KiB pieces; worth ~0.7 %.
