@@ -56,20 +56,23 @@ def _run(cmd, cwd=None):
     return out
 
 
-def build_kernels(verbose: bool = True) -> str:
-    """Each source is compiled to an object of its own (in parallel), then linked."""
+def build_kernels(verbose: bool = True, out: str = None, extra_flags=()) -> str:
+    """Each source is compiled to an object of its own (in parallel), then linked.  `out` and
+    `extra_flags` build a tuning variant beside the shipped library (the TTN_* macros at the top of
+    the kernel sources); load it with TELETRON_AMD_LIB=<out>."""
     from concurrent.futures import ThreadPoolExecutor
 
-    obj_dir = os.path.join(LIB_DIR, "obj")
+    out = os.path.abspath(out) if out else LIB_PATH
+    obj_dir = os.path.join(LIB_DIR, "obj") if out == LIB_PATH else out + ".obj"
     os.makedirs(obj_dir, exist_ok=True)
     objs = [os.path.join(obj_dir, os.path.splitext(src)[0] + ".o") for src in KERNEL_SOURCES]
     with ThreadPoolExecutor(max_workers=min(4, len(KERNEL_SOURCES))) as pool:
-        logs = list(pool.map(lambda so: _run([HIPCC, *HIP_FLAGS, "-c", so[0], "-o", so[1]], cwd=CSRC),
+        logs = list(pool.map(lambda so: _run([HIPCC, *HIP_FLAGS, *extra_flags, "-c", so[0], "-o", so[1]], cwd=CSRC),
                              zip(KERNEL_SOURCES, objs)))
-    logs.append(_run([HIPCC, "--offload-arch=" + ARCH, "-fPIC", "-shared", "-o", LIB_PATH] + objs))
+    logs.append(_run([HIPCC, "--offload-arch=" + ARCH, "-fPIC", "-shared", "-o", out] + objs))
     if verbose:
-        print("built", os.path.relpath(LIB_PATH, ROOT), "\n".join(l for l in logs if l.strip()).strip())
-    return LIB_PATH
+        print("built", os.path.relpath(out, ROOT), "\n".join(l for l in logs if l.strip()).strip())
+    return out
 
 
 def ext_path(name: str) -> str:
@@ -110,4 +113,14 @@ def build_all(verbose: bool = True):
 
 
 if __name__ == "__main__":
-    build_all()
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--variant", metavar="LIB.so", help="build only the kernel library, to this path")
+    ap.add_argument("--flag", action="append", default=[], metavar="-DTTN_...=V",
+                    help="extra hipcc flag for the variant (repeatable)")
+    a = ap.parse_args()
+    if a.variant:
+        build_kernels(out=a.variant, extra_flags=a.flag)
+    else:
+        build_all()

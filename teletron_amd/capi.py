@@ -12,7 +12,10 @@ from typing import Optional
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libteletron_norm.so")
+# TELETRON_AMD_LIB=<path> loads another build of the library (a tuning variant from
+# `python -m teletron_amd.build --variant`); the extension modules always link the shipped one.
+_LIB_PATH = os.environ.get("TELETRON_AMD_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
+                                                               "libteletron_norm.so")
 
 BF16, F32, F16 = 0, 1, 2
 _DTYPES = {torch.bfloat16: BF16, torch.float32: F32, torch.float16: F16}

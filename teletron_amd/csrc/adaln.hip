@@ -62,6 +62,10 @@
 #ifndef TTN_BWD_LOAD_RUNS
 #define TTN_BWD_LOAD_RUNS 1
 #endif
+// 1: a row's first pass waits for the stores of the row before it (see kDrainStores in the kernel)
+#ifndef TTN_BWD_DRAIN_STORES
+#define TTN_BWD_DRAIN_STORES 1
+#endif
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     constexpr int kRowBuffers = (sizeof(T) == 4 && C >= 1024) ? 1 : TTN_ADALN_BWD_ROW_BUFFERS;
     // A row's first pass starts only when the stores of the row before it have left the wavefront
     // (see the RMSNorm backward): 359 us with this wait, 366 us without, at 118 800 rows.
-    constexpr bool kDrainStores = TTN_ADALN_BWD_STORE && !GATED && kRowBuffers == 2 && C >= 1024;
+    constexpr bool kDrainStores = TTN_BWD_DRAIN_STORES && TTN_ADALN_BWD_STORE && !GATED && kRowBuffers == 2 && C >= 1024;
     __shared__ float lds[NSETS * C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;

@@ -34,6 +34,10 @@
 #ifndef TTN_BWD_LOAD_RUNS
 #define TTN_BWD_LOAD_RUNS 1
 #endif
+// 1: a row's first pass waits for the stores of the row before it (see kDrainStores in the kernel)
+#ifndef TTN_BWD_DRAIN_STORES
+#define TTN_BWD_DRAIN_STORES 1
+#endif
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     // of the row before it have left the wavefront (and with them this row's loads, which are older):
     // one wavefront never has more than one row of loads plus one row of stores outstanding.  Measured
     // at 118 800 rows: 354 us with this wait, 365 us when the first pass waits for its loads alone.
-    constexpr bool kDrainStores = TTN_RMS_BWD_STORE && kRowBuffers == 2 && C >= 1024;
+    constexpr bool kDrainStores = TTN_BWD_DRAIN_STORES && TTN_RMS_BWD_STORE && kRowBuffers == 2 && C >= 1024;
     __shared__ float lds[C];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;

@@ -8,6 +8,7 @@ kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for 
         optional <dir>/bench.json                          (the same bench.py run without a profiler)
     python -m teletron_amd.profile_summary workloads --dir gpurun_out/prof     (<dir>/trace_<workload>)
     python -m teletron_amd.profile_summary stream --dir gpurun_out/prof        (<dir>/stream.json, <dir>/stream_stall)
+    python -m teletron_amd.profile_summary variants --dir gpurun_out/prof      (<dir>/variant_<name>.json, _sq, _stall)
 
 The databases are large; run this where they were written and keep only what it writes (--out).
 """
@@ -358,16 +359,95 @@ run faster than it (see bench_cfg4_all_kernels.md).
     print("wrote profiles/stream_ceiling.md")
 
 
+# --------------------------------------------------------------------------------------- variants
+
+VARIANTS = [  # name, build flags, what it changes
+    ("base", "", "the shipped kernels"),
+    ("nodrain", "--flag=-DTTN_BWD_DRAIN_STORES=0",
+     "backward: a row's first pass waits for its own loads only, not for the previous row's stores"),
+    ("plainstore", "--flag=-DTTN_RMS_BWD_STORE=0 --flag=-DTTN_ADALN_BWD_STORE=0",
+     "backward: plain streaming stores instead of write-through"),
+    ("fullahead", "--flag=-DTTN_RMS_BWD_PREFETCH_MID=0 --flag=-DTTN_ADALN_BWD_PREFETCH_MID=0",
+     "backward: the next row is requested before the current one is processed (a full row ahead)"),
+    ("onebuffer", "--flag=-DTTN_RMS_BWD_ROW_BUFFERS=1 --flag=-DTTN_ADALN_BWD_ROW_BUFFERS=1",
+     "backward: one row buffer, no prefetch"),
+    ("twowaves", "--flag=-DTTN_BWD_WAVES_PER_SIMD=2 '--flag=-DTTN_RMS_BWD_BLOCKS_PER_CU=(C>=1024?2:3)' "
+                 "'--flag=-DTTN_ADALN_BWD_BLOCKS_PER_CU=(C>=1024?2:3)'",
+     "backward: two workgroups per compute unit (two wavefronts per SIMD, half the registers each)"),
+    ("fwd5", "'--flag=-DTTN_RMS_FWD_DYN_LDS=(C>=1024?(sizeof(T)==2?0:76800):0)'",
+     "RMSNorm forward: no occupancy throttle (five one-shot workgroups per compute unit instead of three)"),
+]
+
+
+def variants(directory):
+    digest = kernel_source_digest()
+    calls = ["rmsnorm_forward", "rmsnorm_backward", "adaln_forward", "adaln_backward"]
+    rows = ["| variant | ms per step | GB/s | % of 8 TB/s | " + " | ".join(c + " µs" for c in calls) + " |",
+            "|---|---|---|---|" + "---|" * len(calls)]
+    ctr = ["| variant | kernel | SQ_WAIT_INST_ANY | SQ_ACTIVE_INST_ANY | SQ_BUSY_CYCLES | WRREQ_DRAM_CREDIT_STALL | "
+           "RDREQ_DRAM_CREDIT_STALL |", "|---|---|---|---|---|---|---|"]
+    cmds = []
+    for name, flags, what in VARIANTS:
+        bj = os.path.join(directory, f"variant_{name}.json")
+        if not os.path.exists(bj):
+            continue
+        b = json.loads(open(bj).read().strip().splitlines()[-1])
+        rows.append(f"| `{name}` | {b['ms_per_step']:.4f} | {b['value']:.0f} | {100 * b['frac_of_hbm_peak']:.1f} | "
+                    + " | ".join(f"{b['per_call_untimed'][c]['median_us']:.1f}" for c in calls) + " |")
+        cmds.append(f"* `{name}`: {what}" + (f"  \n  `python -m teletron_amd.build --variant /tmp/lib_{name}.so {flags}`" if flags else ""))
+        merged = {}
+        for p in ("sq", "stall"):
+            d = os.path.join(directory, f"variant_{name}_{p}")
+            if os.path.isdir(d):
+                for k, v in counters(d).items():
+                    merged.setdefault(k, {}).update(v)
+        for k, v in sorted(merged.items()):
+            if "bwd_kernel<bf16_t, 3072" in k and "SQ_WAIT_INST_ANY" in v:
+                ctr.append(f"| `{name}` | `{k.split('<')[0]}` | {v['SQ_WAIT_INST_ANY']:,.0f} | {v['SQ_ACTIVE_INST_ANY']:,.0f} | "
+                           f"{v['SQ_BUSY_CYCLES']:,.0f} | {v.get('TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum', float('nan')):,.0f} | "
+                           f"{v.get('TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum', float('nan')):,.0f} |")
+    md = f"""# Tuning variants of the cfg4 step: what each pipeline choice is worth (bench.py, 118 800 x 3072 bf16)
+
+{BOX}.  Kernel sources digest `{digest}`.  Each variant is the shipped kernel source built with other values of
+the tuning macros at the top of `rmsnorm.hip` / `adaln.hip`, loaded in place of the shipped library, and run
+through the unchanged benchmark on one box, one after the other:
+
+    python -m teletron_amd.build --variant /tmp/lib_<name>.so <flags>
+    TELETRON_AMD_LIB=/tmp/lib_<name>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline
+    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY -d gpurun_out/prof/variant_<name>_sq -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum -d gpurun_out/prof/variant_<name>_stall -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+
+{chr(10).join(cmds)}
+
+Per-call figures are HIP-event medians over 30 untimed steps.  Written by
+`python -m teletron_amd.profile_summary variants --dir gpurun_out/prof`.
+
+{chr(10).join(rows)}
+
+Counters of the two backward row kernels, per dispatch (averages):
+
+{chr(10).join(ctr)}
+
+Reading: every alternative keeps more requests in flight per wavefront than the shipped pipeline (or, for
+`onebuffer`, fewer) and is slower; the slower ones show more DRAM-credit stall cycles at the L2-to-memory
+interface, i.e. the extra requests queue instead of being served.  None reaches the 80 % line; see
+stream_ceiling.md for what plain streams of the same read/write mix reach.
+"""
+    with open(os.path.join(PROFILES, "bench_cfg4_tuning_variants.md"), "w") as f:
+        f.write(md)
+    print("wrote bench_cfg4_tuning_variants.md")
+
+
 def main():
     global PROFILES
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=("cfg4", "workloads", "stream"))
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants"))
     ap.add_argument("--dir", default=os.path.join(ROOT, "gpurun_out", "prof"))
     ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
     a = ap.parse_args()
     PROFILES = a.out
     os.makedirs(PROFILES, exist_ok=True)
-    {"cfg4": cfg4, "workloads": workloads, "stream": stream}[a.what](a.dir)
+    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants}[a.what](a.dir)
 
 
 if __name__ == "__main__":
