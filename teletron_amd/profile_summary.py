@@ -2,13 +2,13 @@
 kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for `roofline.kernel` and
 `roofline.traffic`.  Every summary names the commands that produced its inputs.
 
-    python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof
+    python -m teletron_amd.profile_summary cfg4 --dir rocprof_out
         expects  <dir>/trace, <dir>/fetch, <dir>/write   (rocprofv3 -d ... of bench.py, see the text it writes)
         optional <dir>/sq, <dir>/tcc, <dir>/stall          (counter passes)
         optional <dir>/bench.json                          (the same bench.py run without a profiler)
-    python -m teletron_amd.profile_summary workloads --dir gpurun_out/prof     (<dir>/trace_<workload>)
-    python -m teletron_amd.profile_summary stream --dir gpurun_out/prof        (<dir>/stream.json, <dir>/stream_stall)
-    python -m teletron_amd.profile_summary variants --dir gpurun_out/prof      (<dir>/variant_<name>.json, _sq, _stall)
+    python -m teletron_amd.profile_summary workloads --dir rocprof_out     (<dir>/trace_<workload>)
+    python -m teletron_amd.profile_summary stream --dir rocprof_out        (<dir>/stream.json, <dir>/stream_stall)
+    python -m teletron_amd.profile_summary variants --dir rocprof_out      (<dir>/variant_<name>.json, _sq, _stall)
 
 The databases are large; run this where they were written and keep only what it writes (--out).
 """
@@ -24,6 +24,7 @@ import sqlite3
 from teletron_amd.build import ROOT, kernel_source_digest
 
 PROFILES = os.path.join(ROOT, "profiles")
+DIR_SHOWN = "rocprof_out"   # the --dir argument as typed: what the summaries print in their commands
 OURS = ("rmsnorm_", "adaln_", "stream_copy", "stream_probe", "colreduce")
 BOX = "MI355X (gfx950, 256 CUs), ROCm 7.2, one GPU"
 
@@ -161,11 +162,11 @@ Workload: one step = fused RMSNorm(3072) fwd+bwd + fused AdaLN fwd+bwd, through 
 `roofline.traffic` only while the sources it runs have this digest).  rocprofv3 writes a rocpd sqlite database;
 the tables are `select ... from kernels group by name` / `from counters_collection group by kernel_name` over it
 (durations in microseconds, counters in KiB per dispatch as rocprofv3 reports them).  Written by
-`python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof`.
+`python -m teletron_amd.profile_summary cfg4 --dir {DIR_SHOWN}`.
 
 ## Kernel trace
 
-    rocprofv3 --kernel-trace --stats -d gpurun_out/prof/trace -o bench -- {BENCH_CMD.format(steps=30, warmup=5)}
+    rocprofv3 --kernel-trace --stats -d {DIR_SHOWN}/trace -o bench -- {BENCH_CMD.format(steps=30, warmup=5)}
 
 ```
 {stats_table(trace)}
@@ -173,8 +174,8 @@ the tables are `select ... from kernels group by name` / `from counters_collecti
 {bench_note}
 ## HBM traffic (two separate counter runs)
 
-    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/fetch -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
-    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/write -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
+    rocprofv3 --pmc FETCH_SIZE -d {DIR_SHOWN}/fetch -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
+    rocprofv3 --pmc WRITE_SIZE -d {DIR_SHOWN}/write -o bench -- {BENCH_CMD.format(steps=3, warmup=1)}
 
 ```
 {pmc_rows(fetch, 'FETCH_SIZE')}
@@ -218,7 +219,7 @@ def cfg4_counters(passes, digest):
     order.append(next((k for k in merged if k.startswith("stream_copy_kernel")), None))
     order = [k for k in order if k]
     names = [c for p in passes for c in PASS_COUNTERS[p].split()]
-    cmds = "\n".join(f"    rocprofv3 --pmc {PASS_COUNTERS[p]} -d gpurun_out/prof/{p} -o r -- "
+    cmds = "\n".join(f"    rocprofv3 --pmc {PASS_COUNTERS[p]} -d {DIR_SHOWN}/{p} -o r -- "
                      f"{BENCH_CMD.format(steps=3, warmup=1)}" for p in passes)
     lines = ["| counter | " + " | ".join(k.split("<")[0] for k in order) + " |", "|---|" + "---|" * len(order)]
     for c in names:
@@ -236,7 +237,7 @@ def cfg4_counters(passes, digest):
 
 {BOX}.  Kernel sources digest `{digest}`.  Separate counter runs of the same command (rocprofv3 does not split
 counters over passes); values are per dispatch, averaged over the dispatches of the run.  Written by
-`python -m teletron_amd.profile_summary cfg4 --dir gpurun_out/prof`.
+`python -m teletron_amd.profile_summary cfg4 --dir {DIR_SHOWN}`.
 
 {cmds}
 
@@ -281,13 +282,13 @@ def workloads(directory):
 database rocprofv3 wrote (durations in microseconds; torch's own fill/copy kernels of the set-up omitted).
 `stream_copy_kernel` is the copy yardstick over one tensor of the workload (1 read + 1 write).  The JSON line is
 bench.py's own (back-to-back) result for the same command without a profiler, where one was recorded.  Written by
-`python -m teletron_amd.profile_summary workloads --dir gpurun_out/prof`.
+`python -m teletron_amd.profile_summary workloads --dir {DIR_SHOWN}`.
 """]
     for d in sorted(glob.glob(os.path.join(directory, "trace_*"))):
         if not os.path.isdir(d):
             continue
         w = os.path.basename(d)[len("trace_"):]
-        md.append(f"## {w}: {WORKLOAD_INFO.get(w, '')}\n\n    rocprofv3 --kernel-trace --stats -d gpurun_out/prof/trace_{w} "
+        md.append(f"## {w}: {WORKLOAD_INFO.get(w, '')}\n\n    rocprofv3 --kernel-trace --stats -d {DIR_SHOWN}/trace_{w} "
                   f"-o bench -- {BENCH_CMD.format(steps=30, warmup=5)} --workload {w}\n\n```\n{stats_table(kernel_stats(d))}\n```\n")
         bj = os.path.join(directory, f"bench_{w}.json")
         if os.path.exists(bj):
@@ -327,7 +328,7 @@ def stream(directory):
         stall_md = f"""
 ## Where the mixed streams lose (counter pass over the same probes)
 
-    rocprofv3 --pmc {PASS_COUNTERS['stall']} -d gpurun_out/prof/stream_stall -o r -- python3 bench.py --workload stream-ceiling --steps 3 --warmup 4
+    rocprofv3 --pmc {PASS_COUNTERS['stall']} -d {DIR_SHOWN}/stream_stall -o r -- python3 bench.py --workload stream-ceiling --steps 3 --warmup 4
 
 `stream_probe_kernel<reads, writes, accesses per lane, write-through>`; a grid of 65 536 / 262 144 threads is the
 persistent form (256 / 1024 workgroups), anything larger the one-shot form.  Averages per dispatch.
@@ -339,7 +340,7 @@ persistent form (256 / 1024 workgroups), anything larger the one-shot form.  Ave
 {BOX}.  Kernel sources digest `{digest}`.  `python3 bench.py --workload stream-ceiling --steps {b['steps']} --warmup {b['warmup']}`:
 plain streams over 729.9 MB tensors through the library's probe kernel (`tt_norm_stream_probe`: non-temporal
 16-byte loads, one contiguous run per wavefront and tensor, no arithmetic beyond one add), {b['steps']} launches back
-to back between two events.  Written by `python -m teletron_amd.profile_summary stream --dir gpurun_out/prof`.
+to back between two events.  Written by `python -m teletron_amd.profile_summary stream --dir {DIR_SHOWN}`.
 
 Best per mix: read only {best['read_only']['GB/s']:.0f} GB/s ({100 * best['read_only']['frac_of_peak']:.1f} %), two reads
 {best['two_reads']['GB/s']:.0f} ({100 * best['two_reads']['frac_of_peak']:.1f} %), write only {best['write_only']['GB/s']:.0f}
@@ -414,13 +415,13 @@ through the unchanged benchmark on one box, one after the other:
 
     python -m teletron_amd.build --variant /tmp/lib_<name>.so <flags>
     TELETRON_AMD_LIB=/tmp/lib_<name>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline
-    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY -d gpurun_out/prof/variant_<name>_sq -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
-    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum -d gpurun_out/prof/variant_<name>_stall -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY -d {DIR_SHOWN}/variant_<name>_sq -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum -d {DIR_SHOWN}/variant_<name>_stall -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
 
 {chr(10).join(cmds)}
 
 Per-call figures are HIP-event medians over 30 untimed steps.  Written by
-`python -m teletron_amd.profile_summary variants --dir gpurun_out/prof`.
+`python -m teletron_amd.profile_summary variants --dir {DIR_SHOWN}`.
 
 {chr(10).join(rows)}
 
@@ -439,13 +440,14 @@ stream_ceiling.md for what plain streams of the same read/write mix reach.
 
 
 def main():
-    global PROFILES
+    global PROFILES, DIR_SHOWN
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants"))
-    ap.add_argument("--dir", default=os.path.join(ROOT, "gpurun_out", "prof"))
+    ap.add_argument("--dir", default="rocprof_out", help="where rocprofv3 wrote (its -d arguments' parent)")
     ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
     a = ap.parse_args()
     PROFILES = a.out
+    DIR_SHOWN = a.dir.rstrip("/")
     os.makedirs(PROFILES, exist_ok=True)
     {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants}[a.what](a.dir)
 
