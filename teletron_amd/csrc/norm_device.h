@@ -354,6 +354,11 @@ __device__ __forceinline__ void row_pipeline(int64_t grp, int64_t groups, int64_
     }
 }
 
+// Consecutive groups a wavefront takes per step over a strided view of narrow rows (see Strided3Rows)
+#ifndef TTN_STRIDED_RUN
+#define TTN_STRIDED_RUN 6
+#endif
+
 // ---- where a wavefront's rows live ---------------------------------------------
 // A row map turns (wavefront group index, row within the wavefront) into the
 // row's logical number -- its index in the contiguous tensors (out, dout) and in
@@ -369,6 +374,7 @@ struct RowAddr {
 
 // Row-major contiguous [rows, C].
 struct DenseRows {
+    static constexpr int kRun = 1;
     int64_t rows;
     template <int RPW>
     __device__ __forceinline__ int64_t groups() const { return (rows + RPW - 1) / RPW; }
@@ -392,9 +398,21 @@ struct DenseRows {
 // take consecutive i1 for the same i2 tile, so the workgroups running at the
 // same time read neighbouring pieces of the strided side.
 struct Strided3Rows {
+    // Narrow rows: a wavefront takes kRun consecutive groups at a time.  Consecutive groups are consecutive
+    // i1 of one (i0, i2 tile), so when n1 is a multiple of kRun the run needs the divisions of locate() once
+    // (they cost more than a 128-column row itself) and its groups share whatever is indexed by i2 alone.
+    static constexpr int kRun = TTN_STRIDED_RUN;
     int64_t n0, n1, n2;
     int64_t xs0, xs1, xs2;
     int64_t ds0, ds1, ds2;
+    __device__ __forceinline__ bool runs_aligned() const { return n1 % kRun == 0; }
+    // the group h places after `a` inside an aligned run: same i0 and i2, i1 + h
+    __device__ __forceinline__ RowAddr next_in_run(RowAddr a, int h) const {
+        a.row += h * n2;
+        a.xoff += h * xs1;
+        a.doff += h * ds1;
+        return a;
+    }
     template <int RPW>
     __device__ __forceinline__ int64_t groups() const { return n0 * n1 * ((n2 + RPW - 1) / RPW); }
     template <int RPW>

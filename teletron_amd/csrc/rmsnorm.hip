@@ -79,6 +79,33 @@ __device__ __forceinline__ void load_fp32_run(float (&dst)[VEC], const float *p)
     }
 }
 
+// Groups a wavefront takes per step: runs only pay where the index arithmetic and the shared side tables
+// weigh against the row itself, i.e. for narrow rows.
+// Forward without tables: single groups stream better (74 vs 77 us at 712 800 x 128), the divisions hide
+// behind the loads of a kernel that has four times the wavefronts of the backward one.
+template <int C, typename Map, bool SHARES_TABLES = true>
+constexpr int run_length() { return (C < 1024 && SHARES_TABLES) ? Map::kRun : 1; }
+
+// One row's share of the tables in registers: lane l holds the VEC columns of each of its CHUNKS pieces.
+template <bool ON, int CHUNKS, int VEC>
+struct RopeRows {};
+template <int CHUNKS, int VEC>
+struct RopeRows<true, CHUNKS, VEC> {
+    float c[CHUNKS][VEC], s[CHUNKS][VEC];
+    bool on;  // this lane's row is rotated (a row that exists, at a token index below rope.tokens)
+    __device__ __forceinline__ void fetch(const RopeTable &rope, bool ok, int64_t seq, int C, int l, int LANES) {
+        on = ok && seq < rope.tokens;
+        if (on) {
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+                const int64_t col0 = seq * C + (k * LANES + l) * VEC;
+                load_fp32_run<VEC>(c[k], rope.cos + col0);
+                load_fp32_run<VEC>(s[k], rope.sin + col0);
+            }
+        }
+    }
+};
+
 // y -> y*cos + rotate_pairs(y)*sin in fp32 (y already rounded to the element type)
 template <int VEC>
 __device__ __forceinline__ void rotate_pairs_forward(float (&v)[VEC], const float (&c)[VEC], const float (&s)[VEC]) {
@@ -127,54 +154,81 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) wr[k] = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
 
+    // Narrow rows of a strided view: a wavefront takes kRun consecutive groups (see Strided3Rows).  In the
+    // rotary form these are the heads of one token tile, which all read the same rows of the tables: fetched
+    // per row, 1 KiB of table per 256-byte row would make the vector memory pipeline (64 bytes per clock per
+    // compute unit), not HBM, the limit.
+    constexpr int kRun = run_length<C, Map, Rope::kOn>();
     const int64_t groups = map.template groups<RPW>();
-    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
-    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave; grp < groups; grp += stride) {
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves * kRun;
+    [[maybe_unused]] bool aligned = false;
+    if constexpr (kRun > 1) aligned = map.runs_aligned();
+    for (int64_t first = ((int64_t)blockIdx.x * kRowWaves + wave) * kRun; first < groups; first += stride) {
         keep_packed(wr);
-        const RowAddr at = map.template locate<RPW>(grp, sub, C);
-        const int64_t row = at.row;
-        const bool ok = at.ok;
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(x + at.xoff) + l;
-        u32x4 xr[CHUNKS];
+        RowAddr at[kRun];
+        if constexpr (kRun > 1) {
+            if (aligned) {
+                const RowAddr head = map.template locate<RPW>(first, sub, C);
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k) xr[k] = ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
-
-        float ss = 0.0f;
+                for (int h = 0; h < kRun; ++h) at[h] = map.next_in_run(head, h);
+            } else {
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k) {
-            float v[VEC];
-            E::unpack(xr[k], v);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) ss = fmaf(v[j], v[j], ss);
-        }
-        ss = group_sum<LANES>(ss);
-        const float r = 1.0f / sqrtf(ss / (float)C + eps);
-        if (ok && l == 0) rstd[row] = r;
-
-        // the wavefront's rows are consecutive in out: base = its first row
-        const int64_t row0 = map.template locate<RPW>(grp, 0, C).row;
-        const RowWriter<TTN_RMS_FWD_STORE> wo(out + row0 * C, (uint32_t)((sub * C) * sizeof(T)) + l * 16);
-#pragma unroll
-        for (int k = 0; k < CHUNKS; ++k) {
-            float v[VEC], wv[VEC];
-            E::unpack(xr[k], v);
-            E::unpack(wr[k], wv);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] *= r;
-            E::round(v);
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
-            if constexpr (Rope::kOn) {
-                if (ok && at.seq < rope.tokens) {
-                    float cv[VEC], sv[VEC];
-                    const int64_t col0 = at.seq * C + (k * LANES + l) * VEC;
-                    load_fp32_run<VEC>(cv, rope.cos + col0);
-                    load_fp32_run<VEC>(sv, rope.sin + col0);
-                    E::round(v);  // the norm's output in the element type, which the rotation reads
-                    rotate_pairs_forward<VEC>(v, cv, sv);
+                for (int h = 0; h < kRun; ++h) {
+                    at[h] = map.template locate<RPW>(first + h, sub, C);
+                    at[h].ok = at[h].ok && first + h < groups;
                 }
             }
-            if (ok) wo.put(k * LANES, E::pack(v));
+        } else {
+            at[0] = map.template locate<RPW>(first, sub, C);
+        }
+        u32x4 xr[kRun][CHUNKS];
+#pragma unroll
+        for (int h = 0; h < kRun; ++h) {
+            const u32x4 *px = reinterpret_cast<const u32x4 *>(x + at[h].xoff) + l;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) xr[h][k] = at[h].ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        }
+        RopeRows<Rope::kOn, CHUNKS, VEC> rot;
+#pragma unroll
+        for (int h = 0; h < kRun; ++h) {
+            const bool ok = at[h].ok;
+            if constexpr (Rope::kOn) {
+                // the tables depend on the token index alone: fetched when it changes
+                if (h == 0 || at[h].seq != at[h - 1].seq || !rot.on) rot.fetch(rope, ok, at[h].seq, C, l, LANES);
+            }
+            float ss = 0.0f;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+                float v[VEC];
+                E::unpack(xr[h][k], v);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) ss = fmaf(v[j], v[j], ss);
+            }
+            ss = group_sum<LANES>(ss);
+            const float r = 1.0f / sqrtf(ss / (float)C + eps);
+            if (ok && l == 0) rstd[at[h].row] = r;
+
+            // the wavefront's rows are consecutive in out: base = its first row
+            const int64_t row0 = wave_uniform(at[h].row - sub);
+            const RowWriter<TTN_RMS_FWD_STORE> wo(out + row0 * C, (uint32_t)((sub * C) * sizeof(T)) + l * 16);
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) {
+                float v[VEC], wv[VEC];
+                E::unpack(xr[h][k], v);
+                E::unpack(wr[k], wv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[j] *= r;
+                E::round(v);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+                if constexpr (Rope::kOn) {
+                    if (rot.on) {
+                        E::round(v);  // the norm's output in the element type, which the rotation reads
+                        rotate_pairs_forward<VEC>(v, rot.c[k], rot.s[k]);
+                    }
+                }
+                if (ok) wo.put(k * LANES, E::pack(v));
+            }
         }
     }
 }
@@ -237,11 +291,43 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         int64_t seq;     // token index (rotary form only)
         bool ok;
     };
-    auto fetch = [&](RowRegs &b, int64_t grp) {
-        const RowAddr at = map.template locate<RPW>(grp, sub, C);
+    // Narrow rows of a strided view: a wavefront walks runs of kRun consecutive groups (see Strided3Rows and
+    // the forward kernel); the rotary form keeps the table rows it fetched until the token changes.
+    constexpr int kRun = run_length<C, Map>();
+    const int64_t groups = map.template groups<RPW>();
+    const int64_t waves = (int64_t)gridDim.x * kRowWaves;
+    const int64_t me = (int64_t)blockIdx.x * kRowWaves + wave;
+    [[maybe_unused]] bool aligned = false;
+    if constexpr (kRun > 1) aligned = map.runs_aligned();
+    [[maybe_unused]] RowAddr run_head, run_head0;  // first group of the current aligned run: this lane's row, the wavefront's first row
+    [[maybe_unused]] RopeRows<Rope::kOn, CHUNKS, VEC> rot;
+    [[maybe_unused]] int64_t rot_seq = -1;
+    // kRun == 1: at_step is the group.  Otherwise it is the wavefront's own step counter and fetch is called
+    // with 0, 1, 2, ... in turn: step s is place s % kRun of the wavefront's run number s / kRun.
+    auto fetch = [&](RowRegs &b, int64_t at_step) {
+        RowAddr at, at0;
+        if constexpr (kRun == 1) {
+            at = map.template locate<RPW>(at_step, sub, C);
+            at0 = map.template locate<RPW>(at_step, 0, C);
+        } else {
+            const int h = (int)(at_step % kRun);
+            const int64_t first = ((at_step / kRun) * waves + me) * kRun;
+            if (aligned) {
+                if (h == 0) {
+                    run_head = map.template locate<RPW>(first, sub, C);
+                    run_head0 = map.template locate<RPW>(first, 0, C);
+                }
+                at = map.next_in_run(run_head, h);
+                at0 = map.next_in_run(run_head0, h);
+            } else {
+                at = map.template locate<RPW>(first + h, sub, C);
+                at.ok = at.ok && first + h < groups;
+                at0 = map.template locate<RPW>(first + h, 0, C);
+            }
+        }
         b.ok = at.ok;
         b.seq = at.seq;
-        b.doff0 = map.template locate<RPW>(grp, 0, C).doff;
+        b.doff0 = at0.doff;
         b.dlane = (uint32_t)((at.doff - b.doff0) * (int64_t)sizeof(T)) + l * 16;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
@@ -263,15 +349,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         const float r = b.r;
         if constexpr (Rope::kOn) {
             // dout arrives as the gradient of the rotated output: back through the rotation first
-            if (b.ok && b.seq < rope.tokens) {
+            if (b.seq != rot_seq) {
+                rot.fetch(rope, b.ok, b.seq, C, l, LANES);
+                rot_seq = rot.on ? b.seq : -1;
+            }
+            if (b.ok && rot.on) {
 #pragma unroll
                 for (int k = 0; k < CHUNKS; ++k) {
-                    float gv[VEC], cv[VEC], sv[VEC];
-                    const int64_t col0 = b.seq * C + (k * LANES + l) * VEC;
-                    load_fp32_run<VEC>(cv, rope.cos + col0);
-                    load_fp32_run<VEC>(sv, rope.sin + col0);
+                    float gv[VEC];
                     E::unpack(b.g[k], gv);
-                    rotate_pairs_backward<E, VEC>(gv, cv, sv);
+                    rotate_pairs_backward<E, VEC>(gv, rot.c[k], rot.s[k]);
                     b.g[k] = E::pack(gv);
                 }
             }
@@ -327,10 +414,14 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         }
     };
 
-    const int64_t groups = map.template groups<RPW>();
-    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
-    int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave;
-    row_pipeline<kRowBuffers, TTN_RMS_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
+    if constexpr (kRun == 1) {
+        row_pipeline<kRowBuffers, TTN_RMS_BWD_PREFETCH_MID != 0, RowRegs>(me, groups, waves, fetch, process);
+    } else {
+        // runs this wavefront starts: m = 0, 1, ... with (m * waves + me) * kRun < groups
+        const int64_t all_runs = (groups + kRun - 1) / kRun;
+        const int64_t my_runs = all_runs > me ? (all_runs - me + waves - 1) / waves : 0;
+        row_pipeline<kRowBuffers, TTN_RMS_BWD_PREFETCH_MID != 0, RowRegs>(0, my_runs * kRun, 1, fetch, process);
+    }
     flush_column_partials<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds);
 }
 
@@ -360,7 +451,7 @@ static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return st;
-    const RowPlan p = make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kFwdBlocksPerCu, cus);
+    const RowPlan p = make_row_plan(1, rows, RowGeom<T, C>::RPW * run_length<C, Map, Rope::kOn>(), RmsTune<T, C>::kFwdBlocksPerCu, cus);
     if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "rmsnorm forward: grid too large");
     {
         RowKernelProfile prof(stream);

@@ -508,7 +508,7 @@ def _qkv_views(B, S, H, D, dtype, seed, device):
     return q_cpu.transpose(1, 2), k_cpu.transpose(1, 2), q_g.transpose(1, 2), k_g.transpose(1, 2)
 
 
-@pytest.mark.parametrize("B,S,H", [(1, 1001, 24), (2, 37, 6), (1, 3, 1)])
+@pytest.mark.parametrize("B,S,H", [(1, 1001, 24), (2, 37, 6), (1, 3, 1), (1, 129, 13), (2, 4001, 10)])
 def test_rmsnorm_strided_qk_view_matches_eager(capi, gpu_device, B, S, H):
     D = 128
     q_cpu, k_cpu, q_g, k_g = _qkv_views(B, S, H, D, torch.bfloat16, 5, gpu_device)
@@ -534,7 +534,8 @@ def test_rmsnorm_strided_qk_view_matches_eager(capi, gpu_device, B, S, H):
 
 # ------------------------------- rotary embedding fused behind the strided QK-norm
 
-@pytest.mark.parametrize("B,S,H,n_rot", [(1, 1001, 24, 1001), (2, 37, 6, 20), (1, 5, 1, 0), (1, 300, 3, 299), (1, 4, 2, 3)])
+@pytest.mark.parametrize("B,S,H,n_rot", [(1, 1001, 24, 1001), (2, 37, 6, 20), (1, 5, 1, 0), (1, 300, 3, 299), (1, 4, 2, 3),
+                                          (1, 50, 7, 50), (2, 4001, 10, 3999), (3, 2049, 12, 2049)])
 def test_rmsnorm_rope_strided_vs_eager(capi, gpu_device, B, S, H, n_rot):
     """q_layernorm / k_layernorm on the transposed views, then apply_rotary_emb on the first n_rot tokens
     (dit_attention.py:266-273, :435-443), as one kernel each way, against the eager sequence."""
