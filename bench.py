@@ -65,7 +65,8 @@ WORKLOADS = {
                           "contiguous copy, dense RMSNorm Function per tensor, torch.split's backward; same "
                           "traffic accounting as qkv-site (12 slice-sized tensors of useful work)",
     "stream-ceiling": "plain streams over 729.9 MB tensors: 0-2 tensors read, 0-1 written, 1/2/6 KiB per wavefront per "
-                      "tensor, one-shot and persistent grids, streaming and write-through stores; plus the runtime's "
+                      "tensor, one-shot and persistent grids, streaming and write-through stores; the 3+1, 2+2 and 4+2 "
+                      "mixes of the residual and gated kernels; plus the runtime's "
                       "and PyTorch's copies (no normalization arithmetic: the bandwidth envelope the kernels live in)",
     "qkv-site-rope": "the QK-norm call site including the rotary embedding the attention forward applies to q and k "
                      "behind the norms (fp32 cos/sin tables [29700, 128]): QKVSplitNormFunction with the tables, "
@@ -276,9 +277,10 @@ def stream_ceiling(args, torch, capi, dev):
     copy and a PyTorch elementwise copy.  Every figure is back-to-back launches between two events."""
     L = capi.lib()
     nbytes = ROWS * COLS * 2
-    a = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
-    b = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
-    d = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    # two tensors per allocation: the probe's third and fourth read and its second write follow the first
+    a = torch.empty(2 * nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    b = torch.empty(2 * nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    d = torch.empty(2 * nbytes, dtype=torch.uint8, device=dev)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     hip = ctypes.CDLL("libamdhip64.so")
@@ -314,11 +316,22 @@ def stream_ceiling(args, torch, capi, dev):
                               "grid": "one-shot" if blocks == 0 else f"persistent {blocks} workgroups",
                               "store": "write-through" if through else ("streaming" if writes else "-")})
                     rows.append(r)
+    # the mixes of the residual (3 + 1) and gated kernels (forward 2 + 2, backward 4 + 2)
+    for reads, writes in ((3, 1), (2, 2), (4, 2)):
+        for per_lane in (1, 6):
+            for blocks in (0, 256, 1024):
+                for through in (0, 1):
+                    r = probe(reads, writes, per_lane, blocks, through)
+                    r.update({"reads": reads, "writes": writes, "KiB_per_wavefront_per_tensor": per_lane,
+                              "grid": "one-shot" if blocks == 0 else f"persistent {blocks} workgroups",
+                              "store": "write-through" if through else "streaming"})
+                    rows.append(r)
+    d1, a1 = d[:nbytes], a[:nbytes]
     others = {
         "hipMemcpyDtoDAsync": timed(lambda: hip.hipMemcpyDtoDAsync(p(d), p(a), ctypes.c_size_t(nbytes), stream), 2),
-        "torch copy_ (bf16)": timed(lambda: d.view(torch.bfloat16).copy_(a.view(torch.bfloat16)), 2),
-        "torch zero_ (write only)": timed(lambda: d.view(torch.bfloat16).zero_(), 1),
-        "tt_norm_stream_copy": timed(lambda: capi.stream_copy(d, a), 2),
+        "torch copy_ (bf16)": timed(lambda: d1.view(torch.bfloat16).copy_(a1.view(torch.bfloat16)), 2),
+        "torch zero_ (write only)": timed(lambda: d1.view(torch.bfloat16).zero_(), 1),
+        "tt_norm_stream_copy": timed(lambda: capi.stream_copy(d1, a1), 2),
     }
     best = lambda r_, w_: max((r for r in rows if r["reads"] == r_ and r["writes"] == w_), key=lambda r: r["GB/s"])
     two_one = best(2, 1)
@@ -329,7 +342,8 @@ def stream_ceiling(args, torch, capi, dev):
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": WORKLOADS["stream-ceiling"], "tensor_bytes": nbytes},
         "best": {"read_only": best(1, 0), "two_reads": best(2, 0), "write_only": best(0, 1),
-                 "copy_1R_1W": best(1, 1), "2R_1W": two_one},
+                 "copy_1R_1W": best(1, 1), "2R_1W": two_one, "3R_1W": best(3, 1), "2R_2W": best(2, 2),
+                 "4R_2W": best(4, 2)},
         "probes": rows, "other_copies": others,
     }))
 

@@ -281,14 +281,17 @@ int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event);
  * yardstick the benchmark prints next to each result. */
 int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
 
-/* Measurement only (no counterpart in the reference): a plain stream of `reads` tensors read (0..2: a,
- * then b) and `writes` tensors written (0..1: dst), `bytes` each, where every wavefront moves one
- * contiguous run of accesses_per_lane KiB per tensor (1, 2 or 6 accesses of 16 bytes per lane; 6 is
- * the shape of a 3072-column two-byte row).  persistent_blocks = 0 launches one wavefront per run
- * (one-shot grid), otherwise that many workgroups of four wavefronts stride over the runs.
- * write_through != 0 uses the write-through store of the backward kernels.  The benchmark uses it
- * to print what the memory system gives each read/write mix next to the kernels' own figures.
- * The event pair armed by tt_norm_profile_next_row_kernel brackets this kernel as well. */
+/* Measurement only (no counterpart in the reference): a plain stream of `reads` tensors read and `writes`
+ * tensors written, `bytes` each, where every wavefront moves one contiguous run of accesses_per_lane KiB
+ * per tensor (1, 2 or 6 accesses of 16 bytes per lane; 6 is the shape of a 3072-column two-byte row).
+ * Tensors read: a, b, a + bytes, b + bytes (reads 0..4); written: dst, dst + bytes (writes 0..2) -- the
+ * allocations must be that long.  Built mixes: up to 2 reads with up to 1 write in every shape; 3+1, 2+2
+ * and 4+2 (the mixes of the residual and gated kernels) with 1 and 6 accesses per lane.
+ * persistent_blocks = 0 launches one wavefront per run (one-shot grid), otherwise that many workgroups
+ * of four wavefronts stride over the runs.  write_through != 0 uses the write-through store of the
+ * backward kernels.  The benchmark uses it to print what the memory system gives each read/write mix
+ * next to the kernels' own figures.  The event pair armed by tt_norm_profile_next_row_kernel brackets
+ * this kernel as well. */
 int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
                          int accesses_per_lane, int persistent_blocks, int write_through, void *stream);
 

@@ -178,37 +178,46 @@ __global__ __launch_bounds__(kRowThreads) void stream_copy_kernel(u32x4 *__restr
 
 // ---- streaming probe -----------------------------------------------------------
 // Plain streams with the access shapes the row kernels can choose from, for measuring what this
-// memory system gives each read/write mix: NR tensors read (0, 1 or 2), NW written (0 or 1);
+// memory system gives each read/write mix: NR tensors read (0..4), NW written (0..2);
 // every wavefront moves one contiguous run of D KiB per tensor (D 16-byte accesses per lane; 6 is
 // a 3072-column two-byte row) and either exits (one-shot grid) or strides on (persistent grid).
 // Loads carry the non-temporal hint; THROUGH picks the store (see RowWriter).
+struct ProbeTensors {
+    const u32x4 *read[4];
+    u32x4 *write[2];
+};
+
 template <int NR, int NW, int D, int THROUGH>
-__global__ __launch_bounds__(kRowThreads) void stream_probe_kernel(u32x4 *__restrict__ dst,
-                                                                   const u32x4 *__restrict__ a,
-                                                                   const u32x4 *__restrict__ b, int64_t runs,
+__global__ __launch_bounds__(kRowThreads) void stream_probe_kernel(const ProbeTensors t, int64_t runs,
                                                                    u32x4 *__restrict__ sink) {
     const int lane = threadIdx.x & 63;
     u32x4 keep{0, 0, 0, 0};
     const int64_t stride = (int64_t)gridDim.x * kRowWaves;
     for (int64_t run = (int64_t)blockIdx.x * kRowWaves + wave_id_in_block(); run < runs; run += stride) {
         const int64_t at = run * (D * kWaveSize);
-        u32x4 v[D];
+        u32x4 v[NR > 0 ? NR : 1][D];
+        if constexpr (NR == 0) {
 #pragma unroll
-        for (int k = 0; k < D; ++k) v[k] = NR >= 1 ? load16_stream(a + at + lane + k * kWaveSize) : u32x4{(uint32_t)run, 1, 2, 3};
-        if constexpr (NR >= 2) {
-            u32x4 w[D];
-#pragma unroll
-            for (int k = 0; k < D; ++k) w[k] = load16_stream(b + at + lane + k * kWaveSize);
-#pragma unroll
-            for (int k = 0; k < D; ++k) v[k] += w[k];
+            for (int k = 0; k < D; ++k) v[0][k] = u32x4{(uint32_t)run, 1, 2, 3};
         }
-        if constexpr (NW >= 1) {
-            const RowWriter<THROUGH> wr(dst + at, lane * 16);
 #pragma unroll
-            for (int k = 0; k < D; ++k) wr.put(k * kWaveSize, v[k]);
+        for (int i = 0; i < NR; ++i)
+#pragma unroll
+            for (int k = 0; k < D; ++k) v[i][k] = load16_stream(t.read[i] + at + lane + k * kWaveSize);
+#pragma unroll
+        for (int i = 1; i < NR; ++i)
+#pragma unroll
+            for (int k = 0; k < D; ++k) v[0][k] += v[i][k];
+        if constexpr (NW >= 1) {
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                const RowWriter<THROUGH> wr(t.write[j] + at, lane * 16);
+#pragma unroll
+                for (int k = 0; k < D; ++k) wr.put(k * kWaveSize, v[0][k] + (uint32_t)j);
+            }
         } else {
 #pragma unroll
-            for (int k = 0; k < D; ++k) keep += v[k];
+            for (int k = 0; k < D; ++k) keep += v[0][k];
         }
     }
     // read-only probes: keep the loads alive without ever storing
@@ -216,11 +225,9 @@ __global__ __launch_bounds__(kRowThreads) void stream_probe_kernel(u32x4 *__rest
 }
 
 template <int NR, int NW, int D, int THROUGH>
-static int launch_stream_probe(void *dst, const void *a, const void *b, int64_t runs, int64_t blocks,
-                               hipStream_t stream) {
+static int launch_stream_probe(const ProbeTensors &t, int64_t runs, int64_t blocks, hipStream_t stream) {
     RowKernelProfile prof(stream);
-    stream_probe_kernel<NR, NW, D, THROUGH><<<dim3((unsigned)blocks), dim3(kRowThreads), 0, stream>>>(
-        (u32x4 *)dst, (const u32x4 *)a, (const u32x4 *)b, runs, (u32x4 *)dst);
+    stream_probe_kernel<NR, NW, D, THROUGH><<<dim3((unsigned)blocks), dim3(kRowThreads), 0, stream>>>(t, runs, t.write[0]);
     return TT_NORM_OK;
 }
 
@@ -276,8 +283,8 @@ int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) 
 
 int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
                          int accesses_per_lane, int persistent_blocks, int write_through, void *stream) {
-    if (reads < 0 || reads > 2 || writes < 0 || writes > 1 || reads + writes == 0)
-        return fail(TT_NORM_EINVAL, "stream_probe: reads=%d (0..2) writes=%d (0..1), at least one stream", reads, writes);
+    if (reads < 0 || reads > 4 || writes < 0 || writes > 2 || reads + writes == 0)
+        return fail(TT_NORM_EINVAL, "stream_probe: reads=%d (0..4) writes=%d (0..2), at least one stream", reads, writes);
     if (accesses_per_lane != 1 && accesses_per_lane != 2 && accesses_per_lane != 6)
         return fail(TT_NORM_EUNSUPPORTED, "stream_probe: accesses_per_lane=%d (built for 1, 2 and 6)", accesses_per_lane);
     if (persistent_blocks < 0) return fail(TT_NORM_EINVAL, "stream_probe: persistent_blocks=%d", persistent_blocks);
@@ -291,9 +298,14 @@ int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, 
     if (blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "stream_probe: grid too large");
     const hipStream_t s = (hipStream_t)stream;
     const int through = (write_through && writes) ? 1 : 0;
+    // tensors 3 and 4 read, and the second one written, follow the first ones in the same allocations
+    const char *ca = (const char *)a, *cb = (const char *)b;
+    char *cd = (char *)dst;
+    const ProbeTensors t{{(const u32x4 *)ca, (const u32x4 *)cb, (const u32x4 *)(ca + bytes), (const u32x4 *)(cb + bytes)},
+                         {(u32x4 *)cd, (u32x4 *)(cd + bytes)}};
 #define TTN_PROBE(NR, NW, D, TH)                                                          \
     if (reads == NR && writes == NW && accesses_per_lane == D && through == TH) {         \
-        launch_stream_probe<NR, NW, D, TH>(dst, a, b, runs, blocks, s);                   \
+        launch_stream_probe<NR, NW, D, TH>(t, runs, blocks, s);                           \
         return check_launch("stream probe launch");                                       \
     }
 #define TTN_PROBE_D(NR, NW, TH) TTN_PROBE(NR, NW, 1, TH) TTN_PROBE(NR, NW, 2, TH) TTN_PROBE(NR, NW, 6, TH)
@@ -301,6 +313,11 @@ int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, 
     TTN_PROBE_D(0, 1, 0) TTN_PROBE_D(1, 1, 0) TTN_PROBE_D(2, 1, 0)
     TTN_PROBE_D(0, 1, 1) TTN_PROBE_D(1, 1, 1) TTN_PROBE_D(2, 1, 1)
 #undef TTN_PROBE_D
+    // the mixes of the gated residual kernels (forward 2 reads + 2 writes, backward 4 + 2) and of the
+    // backward with a residual gradient (3 + 1), in the one-row and the 1 KiB shapes
+#define TTN_PROBE_W(NR, NW) TTN_PROBE(NR, NW, 1, 0) TTN_PROBE(NR, NW, 6, 0) TTN_PROBE(NR, NW, 1, 1) TTN_PROBE(NR, NW, 6, 1)
+    TTN_PROBE_W(3, 1) TTN_PROBE_W(2, 2) TTN_PROBE_W(4, 2)
+#undef TTN_PROBE_W
 #undef TTN_PROBE
     return fail(TT_NORM_EUNSUPPORTED, "stream_probe: no kernel for this combination");
 }

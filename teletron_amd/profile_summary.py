@@ -345,7 +345,9 @@ to back between two events.  Written by `python -m teletron_amd.profile_summary 
 Best per mix: read only {best['read_only']['GB/s']:.0f} GB/s ({100 * best['read_only']['frac_of_peak']:.1f} %), two reads
 {best['two_reads']['GB/s']:.0f} ({100 * best['two_reads']['frac_of_peak']:.1f} %), write only {best['write_only']['GB/s']:.0f}
 ({100 * best['write_only']['frac_of_peak']:.1f} %), copy 1R+1W {best['copy_1R_1W']['GB/s']:.0f} ({100 * best['copy_1R_1W']['frac_of_peak']:.1f} %),
-2R+1W {best['2R_1W']['GB/s']:.0f} ({100 * best['2R_1W']['frac_of_peak']:.1f} %).  Pure streams run at 85-92 % of the
+2R+1W {best['2R_1W']['GB/s']:.0f} ({100 * best['2R_1W']['frac_of_peak']:.1f} %), 3R+1W {best['3R_1W']['GB/s']:.0f}
+({100 * best['3R_1W']['frac_of_peak']:.1f} %), 2R+2W {best['2R_2W']['GB/s']:.0f} ({100 * best['2R_2W']['frac_of_peak']:.1f} %), 4R+2W
+{best['4R_2W']['GB/s']:.0f} ({100 * best['4R_2W']['frac_of_peak']:.1f} %).  Pure streams run at 85-92 % of the
 published peak; as soon as reads and writes mix, every shape drops to 72-82 %.  A row kernel moves 6 KiB per
 wavefront and tensor (a whole 3072-column row, which it needs for the row statistics): in that shape the best plain
 2R+1W stream is the one-shot grid, and the backward kernels (persistent, because the column sums live in registers)
