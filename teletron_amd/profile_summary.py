@@ -270,7 +270,11 @@ WORKLOAD_INFO = {
     "cfg3": "AdaLN fwd+bwd, 29 700 x 3072 bf16",
     "cfg5": "AdaLN -> RMSNorm chain, 4 x 11 056 x 3072 bf16, one modulation row per sample",
     "w1536-f16": "any-width kernels: RMSNorm + AdaLN fwd+bwd, 237 600 x 1536 fp16",
+    "qkv-site": "QK-norm call site through the autograd Function: q and k normalised on the strided views of the "
+                "fused QKV projection, gradients written straight into the projection's gradient",
     "qkv-site-rope": "QK-norm call site with the rotary embedding fused behind the norm",
+    "qkv-site-rope-reference": "the same call site the reference's way: split, transposing copy, dense RMSNorm, rotary "
+                               "embedding as PyTorch ops",
 }
 
 
