@@ -130,6 +130,15 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
                                 int64_t cols, int dtype,
                                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* Rows of a contiguous [n0, n1, n2, cols] tensor `src` copied into a strided view `dst` of that shape
+ * (strides in elements, multiples of 16 bytes; contiguous last dimension).  The QK-norm call site's
+ * value gradient: v is a view of the fused projection, so dv [B, H, S, D] belongs in the v slice of the
+ * projection's gradient beside the dq and dk that tt_rmsnorm_backward_strided writes there -- what
+ * torch.split's backward does in the reference by concatenating three separate gradients
+ * (teletron/models/dit/dit_attention.py:149-214).  Any cols that make whole 16-byte pieces. */
+int tt_norm_copy_rows_strided(void *dst, const void *src, int64_t n0, int64_t n1, int64_t n2, int64_t ds0,
+                              int64_t ds1, int64_t ds2, int64_t cols, int dtype, void *stream);
+
 /* The strided QK-norm with the rotary embedding the attention caller applies right behind it
  * (teletron/models/dit/dit_attention.py:266-273 and :435-443: apply_rotary_emb(query, (freqs_cos,
  * freqs_sin)) on the [B, H, S, D] result of q_layernorm / k_layernorm, a separate read + write pass

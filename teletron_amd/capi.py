@@ -30,7 +30,7 @@ EXPORTS = (
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
     "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual", "tt_adaln_backward_static",
     "tt_norm_stream_probe", "tt_rmsnorm_rope_forward_strided", "tt_rmsnorm_rope_backward_strided",
-    "tt_adaln_forward_seq_first", "tt_adaln_backward_seq_first",
+    "tt_adaln_forward_seq_first", "tt_adaln_backward_seq_first", "tt_norm_copy_rows_strided",
 )
 
 
@@ -80,6 +80,7 @@ def lib() -> ctypes.CDLL:
         L.tt_gated_residual_adaln_backward.argtypes = [vp] * 13 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_residual.argtypes = [vp] * 9 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
+        L.tt_norm_copy_rows_strided.argtypes = [vp, vp] + [i64] * 7 + [ci, vp]
         L.tt_norm_stream_probe.argtypes = [vp, vp, vp, sz, ci, ci, ci, ci, ci, vp]
         L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
@@ -194,6 +195,18 @@ def rmsnorm_backward_strided(dout, x, weight, rstd, dx=None):
                                              n0, n1, n2, s0, s1, s2, d0, d1, d2, cols, _dt(x), _p(ws), n,
                                              _stream(x)), "tt_rmsnorm_backward_strided")
     return dx, dweight
+
+
+def copy_rows_strided(dst, src):
+    """src contiguous; dst any view (<= 4-D, contiguous last dim, 16-byte aligned strides) of src's shape."""
+    _dense_gpu(src)
+    if dst.shape != src.shape or dst.dtype != src.dtype or not dst.is_cuda:
+        raise ValueError("dst must be a GPU view of src's shape and dtype")
+    (n0, n1, n2), (d0, d1, d2) = _view3(dst)
+    with torch.cuda.device(src.device):
+        _check(lib().tt_norm_copy_rows_strided(_p(dst), _p(src), n0, n1, n2, d0, d1, d2, src.shape[-1], _dt(src),
+                                               _stream(src)), "tt_norm_copy_rows_strided")
+    return dst
 
 
 def rmsnorm_rope_forward_strided(x, weight, cos, sin, eps: float):

@@ -147,6 +147,22 @@ void torch_launch_rms_backward_strided(torch::Tensor &dinp, torch::Tensor &dweig
              "tt_rmsnorm_backward_strided");
 }
 
+// dst: any view (<= 4-D, contiguous last dimension) of src's shape; src contiguous.  The value gradient of the
+// QK-norm call site goes into its slice of the fused projection's gradient with this.
+void torch_launch_copy_rows_strided(torch::Tensor &dst, const torch::Tensor &src) {
+    const auto dev = src.device();
+    TORCH_CHECK(dst.is_cuda() && dst.device() == dev, "dst and src must be on the same GPU");
+    check_dense_on(src, dev, "src");
+    TORCH_CHECK(dst.sizes() == src.sizes() && dst.scalar_type() == src.scalar_type(), "dst must have src's shape and dtype");
+    const int dt = dtype_code(src, "src");
+    const int64_t cols = src.size(-1);
+    const View3 vd = view3(dst, cols, "dst");
+    c10::DeviceGuard guard(dev);
+    raise_on(tt_norm_copy_rows_strided(dst.data_ptr(), src.data_ptr(), vd.n[0], vd.n[1], vd.n[2], vd.s[0], vd.s[1],
+                                       vd.s[2], cols, dt, current_stream(src)),
+             "tt_norm_copy_rows_strided");
+}
+
 // ---- strided QK-norm with the rotary embedding behind it (no reference counterpart: the reference
 // runs apply_rotary_emb as separate PyTorch ops on the norm's output) ----
 static int64_t check_rope_tables(const torch::Tensor &cos, const torch::Tensor &sin, const at::Device &dev,
@@ -225,6 +241,8 @@ void torch_launch_rms_rope_backward_strided(torch::Tensor &dinp, torch::Tensor &
 }
 
 PYBIND11_MODULE(fused_rmsnorm, m) {
+    m.def("torch_launch_copy_rows_strided", &torch_launch_copy_rows_strided,
+          "rows of a contiguous tensor into a strided view of the same shape");
     m.def("torch_launch_rms_rope_forward_strided", &torch_launch_rms_rope_forward_strided,
           "strided RMSNorm forward with the rotary embedding applied to the result");
     m.def("torch_launch_rms_rope_backward_strided", &torch_launch_rms_rope_backward_strided,

@@ -425,6 +425,32 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     flush_column_partials<G, 1>(acc, partial + (int64_t)blockIdx.x * C, lds);
 }
 
+// ---- rows of a contiguous tensor into a strided view --------------------------
+// The value gradient of the QK-norm call site: v leaves the forward as a view of the fused projection, so its
+// gradient arrives as a contiguous [B, H, S, D] tensor and belongs in the v slice of the projection's
+// gradient, next to the dq and dk the backward kernels write there (torch.split's backward in the reference,
+// teletron/models/dit/dit_attention.py:149-214).  Same traversal as the norm kernels: a wavefront takes
+// 64 / LANES consecutive i2 of one (i0, i1), consecutive wavefronts consecutive i1.  Offsets of `map` count
+// 16-byte pieces; a row is `pieces` of them.
+template <int LANES>
+__global__ __launch_bounds__(kRowThreads) void copy_rows_strided_kernel(u32x4 *__restrict__ dst,
+                                                                        const u32x4 *__restrict__ src,
+                                                                        const Strided3Rows map, int pieces) {
+    constexpr int RPW = kWaveSize / LANES;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LANES;
+    const int l = lane % LANES;
+    const int64_t groups = map.template groups<RPW>();
+    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
+    for (int64_t grp = (int64_t)blockIdx.x * kRowWaves + wave_id_in_block(); grp < groups; grp += stride) {
+        const RowAddr at = map.template locate<RPW>(grp, sub, 0);
+        if (!at.ok) continue;
+        const u32x4 *from = src + at.row * pieces;
+        u32x4 *to = dst + at.doff;
+        for (int p = l; p < pieces; p += LANES) store16_stream(to + p, load16_stream(from + p));
+    }
+}
+
 // ---- tuning: workgroups per compute unit of the persistent grids ------------
 // Forward at 3072 columns runs one-shot (one row per wavefront, then exit; the
 // hardware dispatcher keeps a steady mix of loading and storing wavefronts, which
@@ -640,6 +666,46 @@ int tt_rmsnorm_backward_strided(void *dx, void *dweight, const void *dout, const
                                            workspace_bytes, (hipStream_t)stream)
     TTN_DISPATCH(dtype, cols, CALL);
 #undef CALL
+}
+
+int tt_norm_copy_rows_strided(void *dst, const void *src, int64_t n0, int64_t n1, int64_t n2, int64_t ds0,
+                              int64_t ds1, int64_t ds2, int64_t cols, int dtype, void *stream) {
+    const char *who = "tt_norm_copy_rows_strided";
+    if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F16 && dtype != TT_NORM_F32)
+        return fail(TT_NORM_EUNSUPPORTED, "%s: dtype %d", who, dtype);
+    const int64_t vec = 16 / (int64_t)elem_bytes(dtype);
+    if (cols <= 0 || cols % vec != 0 || cols / vec > (1 << 20))
+        return fail(TT_NORM_EUNSUPPORTED, "%s: cols=%lld is not a whole number of 16-byte pieces", who, (long long)cols);
+    if (n0 < 0 || n1 < 0 || n2 < 0)
+        return fail(TT_NORM_EINVAL, "%s: sizes [%lld, %lld, %lld]", who, (long long)n0, (long long)n1, (long long)n2);
+    for (int64_t s : {ds0, ds1, ds2})
+        if (s < 0 || s % vec != 0)
+            return fail(TT_NORM_EALIGN, "%s: dst stride %lld is not a non-negative multiple of %lld elements (16 bytes)",
+                        who, (long long)s, (long long)vec);
+    const int64_t rows = n0 * n1 * n2;
+    if (rows == 0) return TT_NORM_OK;
+    if (!dst || !src) return fail(TT_NORM_EINVAL, "%s: null pointer", who);
+    if (!aligned16(dst) || !aligned16(src)) return fail(TT_NORM_EALIGN, "%s: pointer not 16-byte aligned", who);
+    int st = TT_NORM_OK;
+    const int cus = current_device_cus(&st);
+    if (st != TT_NORM_OK) return st;
+    const int pieces = (int)(cols / vec);
+    const Strided3Rows map{n0, n1, n2, 0, 0, 0, ds0 / vec, ds1 / vec, ds2 / vec};
+    const int lanes = pieces <= 4 ? 4 : pieces <= 8 ? 8 : pieces <= 16 ? 16 : pieces <= 32 ? 32 : 64;
+    const RowPlan p = make_row_plan(1, rows, kWaveSize / lanes, 16, cus);
+    if (p.blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "%s: grid too large", who);
+    const dim3 grid((unsigned)p.blocks), block(kRowThreads);
+    const hipStream_t s = (hipStream_t)stream;
+    u32x4 *d = (u32x4 *)dst;
+    const u32x4 *f = (const u32x4 *)src;
+    switch (lanes) {
+        case 4: copy_rows_strided_kernel<4><<<grid, block, 0, s>>>(d, f, map, pieces); break;
+        case 8: copy_rows_strided_kernel<8><<<grid, block, 0, s>>>(d, f, map, pieces); break;
+        case 16: copy_rows_strided_kernel<16><<<grid, block, 0, s>>>(d, f, map, pieces); break;
+        case 32: copy_rows_strided_kernel<32><<<grid, block, 0, s>>>(d, f, map, pieces); break;
+        default: copy_rows_strided_kernel<64><<<grid, block, 0, s>>>(d, f, map, pieces); break;
+    }
+    return check_launch("strided row copy launch");
 }
 
 /* ---- strided QK-norm with the rotary embedding applied behind it (head dimension 128) ---- */

@@ -604,7 +604,7 @@ class QKVSplitNormFunction(Function):
         if grad_v is None:
             slices[2].zero_()
         else:
-            slices[2].copy_(grad_v)
+            fused_rmsnorm.torch_launch_copy_rows_strided(slices[2], _aligned_contiguous(grad_v.to(mixed.dtype)))
         return (d_mixed, grads_w[0], grads_w[1], None) + (None,) * ctx.n_rotary
 
 

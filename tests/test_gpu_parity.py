@@ -532,6 +532,44 @@ def test_rmsnorm_strided_qk_view_matches_eager(capi, gpu_device, B, S, H):
         assert torch.equal(dx.contiguous(), dx_dense)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("B,S,H,D", [(1, 1001, 24, 128), (2, 37, 6, 64), (1, 3, 1, 8), (2, 130, 5, 40), (1, 9, 2, 3072)])
+def test_copy_rows_strided_into_the_value_slice(capi, gpu_device, dtype, B, S, H, D):
+    """dv [B, H, S, D] into the v slice of the fused projection's gradient [B, S, H, 3D], bit for bit what
+    Tensor.copy_ writes there, and nothing outside the slice."""
+    gen = torch.Generator().manual_seed(B * 1000 + S)
+    src = torch.randn(B, H, S, D, generator=gen).to(dtype).to(gpu_device)
+    whole = torch.full((B, S, H, 3 * D), 7.0, dtype=dtype, device=gpu_device)
+    want = whole.clone()
+    want[..., 2 * D:].transpose(1, 2).copy_(src)
+    got = capi.copy_rows_strided(whole[..., 2 * D:].transpose(1, 2), src)
+    assert got.data_ptr() == whole[..., 2 * D:].data_ptr()
+    assert torch.equal(whole, want)
+    # a 3-D and a 2-D view, and no rows at all
+    flat = torch.zeros(S * H, 2 * D, dtype=dtype, device=gpu_device)
+    capi.copy_rows_strided(flat[:, D:], src[0].reshape(H * S, D).contiguous())
+    assert torch.equal(flat[:, D:], src[0].reshape(H * S, D)) and not flat[:, :D].any()
+    capi.copy_rows_strided(whole[:0, :, :, :D].transpose(1, 2), src[:0])
+
+
+def test_copy_rows_strided_rejects_what_it_cannot_address(capi, gpu_device):
+    L = capi.lib()
+    buf = torch.zeros(64, 3 * 128 + 4, dtype=torch.bfloat16, device=gpu_device)
+    src = torch.zeros(64, 128, dtype=torch.bfloat16, device=gpu_device)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    # row stride of 388 elements = 776 bytes: not a multiple of 16
+    assert L.tt_norm_copy_rows_strided(p(buf), p(src), 1, 1, 64, 0, 0, 388, 128, capi.BF16, None) == 3
+    # misaligned base, a row that is not whole 16-byte pieces, an unknown dtype
+    ok = torch.zeros(64, 384, dtype=torch.bfloat16, device=gpu_device)
+    assert L.tt_norm_copy_rows_strided(ctypes.c_void_p(ok.data_ptr() + 2), p(src), 1, 1, 64, 0, 0, 384, 128,
+                                       capi.BF16, None) == 3
+    assert L.tt_norm_copy_rows_strided(p(ok), p(src), 1, 1, 64, 0, 0, 384, 100, capi.BF16, None) == 2
+    assert L.tt_norm_copy_rows_strided(p(ok), p(src), 1, 1, 64, 0, 0, 384, 128, 9, None) == 2
+    assert not ok.any()
+    with pytest.raises(ValueError):
+        capi.copy_rows_strided(ok[:, :128], src.float())
+
+
 # ------------------------------- rotary embedding fused behind the strided QK-norm
 
 @pytest.mark.parametrize("B,S,H,n_rot", [(1, 1001, 24, 1001), (2, 37, 6, 20), (1, 5, 1, 0), (1, 300, 3, 299), (1, 4, 2, 3),
