@@ -16,7 +16,9 @@ What differs from the reference, on purpose:
     reference kernels only handle a single modulation row;
   * both operators accept any row of whole 16-byte pieces (up to 8192 two-byte or
     4096 four-byte columns) in bf16, fp16 or fp32; 128 and 3072 columns
-    run the tuned kernels, and only those take strided views or the gated form;
+    run the tuned kernels; strided views are read in place at every width, the
+    gated and residual forms exist for rows of up to 384 pieces, the rotary form
+    for 128 columns;
   * gated_residual_layer_norm fuses the residual update in front of a modulated
     LayerNorm (dit_layerspec.py:152-163) into the norm, forward and backward;
   * nothing here falls back silently: with FUSED_KERNELS on, a missing
