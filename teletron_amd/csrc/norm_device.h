@@ -120,9 +120,15 @@ struct Elem<f16_t> {
         u32x4 r;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            // The value is an fp32 number before it is converted, as in the eager formulas (an fp32 op, then
+            // .to(half)).  Left to itself the compiler folds the producing multiply into a mixed-precision
+            // instruction in some kernels and not in others, and one element in ten thousand then differs
+            // by an ulp from kernel to kernel.
+            float lo = v[2 * i], hi = v[2 * i + 1];
+            asm("" : "+v"(lo), "+v"(hi));
             f16x2_t h;
-            h[0] = (_Float16)v[2 * i];
-            h[1] = (_Float16)v[2 * i + 1];
+            h[0] = (_Float16)lo;
+            h[1] = (_Float16)hi;
             r[i] = __builtin_bit_cast(uint32_t, h);
         }
         return r;

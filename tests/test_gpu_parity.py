@@ -607,6 +607,44 @@ def test_rmsnorm_rope_strided_vs_eager(capi, gpu_device, B, S, H, n_rot):
         assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("B,S,H,n_rot", [(1, 1001, 24, 1001), (2, 131, 5, 100)])
+def test_rmsnorm_strided_and_rope_in_fp16_and_fp32(capi, gpu_device, dtype, B, S, H, n_rot):
+    """The other element types through the strided and the rotary kernels at head dimension 128 (two rows
+    per wavefront in fp32): identities that hold bit for bit whatever the type, and the truth in float64."""
+    D = 128
+    q_cpu, _, q_g, _ = _qkv_views(B, S, H, D, dtype, 25, gpu_device)
+    gen = torch.Generator().manual_seed(26)
+    w = (1 + 0.02 * torch.randn(D, generator=gen)).to(dtype)
+    grad = torch.randn(B, H, S, D, generator=gen).to(dtype)
+    cos, sin = O.make_rope_tables(n_rot, D, seed=S)
+    w_g, grad_g, cos_g, sin_g = w.to(gpu_device), grad.to(gpu_device), cos.to(gpu_device), sin.to(gpu_device)
+    # plain strided norm == dense norm on a materialised copy, forward and backward
+    out, rstd = capi.rmsnorm_forward_strided(q_g, w_g, EPS)
+    out_dense, rstd_dense = capi.rmsnorm_forward(q_g.contiguous(), w_g, EPS)
+    assert torch.equal(out, out_dense) and torch.equal(rstd, rstd_dense)
+    dx, dw = capi.rmsnorm_backward_strided(grad_g, q_g, w_g, rstd)
+    dx_dense, dw_dense = capi.rmsnorm_backward(grad_g, q_g.contiguous(), w_g, rstd_dense)
+    assert torch.equal(dx.contiguous(), dx_dense)
+    torch.testing.assert_close(dw.float(), dw_dense.float(), rtol=2e-3 if dtype == torch.float16 else 1e-5, atol=1e-3)
+    # rotary form: rows past the table are the plain norm; the backward equals "gradient rotated back by
+    # autograd on the host, then the plain strided backward"
+    out_r, rstd_r = capi.rmsnorm_rope_forward_strided(q_g, w_g, cos_g, sin_g, EPS)
+    assert torch.equal(out_r[:, :, n_rot:], out[:, :, n_rot:]) and torch.equal(rstd_r, rstd)
+    dx_r, dw_r = capi.rmsnorm_rope_backward_strided(grad_g, q_g, w_g, rstd, cos_g, sin_g)
+    yl = out.cpu().requires_grad_(True)
+    torch.cat([O.apply_rotary_emb_real(yl[:, :, :n_rot], cos, sin), yl[:, :, n_rot:]], dim=2).backward(grad)
+    dx2, dw2 = capi.rmsnorm_backward_strided(yl.grad.contiguous().to(gpu_device), q_g, w_g, rstd)
+    assert torch.equal(dx_r, dx2) and torch.equal(dw_r, dw2)
+    # against the float64 truth: one rounding of the result in fp32, the element type's grid in fp16
+    t_out, t_dx, t_dw = O.truth_qk_norm_rope_fwd_bwd(q_cpu, w, cos, sin, grad)
+    tol = dict(rtol=4e-3, atol=4e-3) if dtype == torch.float16 else dict(rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(out_r.cpu().double(), t_out, **tol)
+    torch.testing.assert_close(dx_r.cpu().double(), t_dx, **tol)
+    rows = B * H * S
+    torch.testing.assert_close(dw_r.cpu().double(), t_dw, rtol=0, atol=(4e-3 if dtype == torch.float16 else 1e-5) * rows ** 0.5)
+
+
 def test_rmsnorm_rope_rejects_other_head_dims_and_bad_tables(capi, gpu_device):
     x = torch.zeros(1, 2, 8, 3072, dtype=torch.bfloat16, device=gpu_device)
     w = torch.ones(3072, dtype=torch.bfloat16, device=gpu_device)
