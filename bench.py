@@ -51,6 +51,9 @@ WORKLOADS = {
             "fwd+bwd on both (4 C-ABI calls)",
     "cfg2-strided": "cfg2 on the call site's own layout: q and k are transposed [B, H, S, D] views into the fused "
                     "[1, 29700, 24, 384] QKV projection, read in place; outputs and dx contiguous (4 C-ABI calls)",
+    "cfg2-strided-rope": "cfg2-strided with the rotary embedding applied behind each norm (fp32 cos/sin tables "
+                         "[29700, 128], every token rotated), forward and backward (4 C-ABI calls; the tables' bytes "
+                         "are not counted)",
     "cfg3": "cfg3: 29700 tokens x 3072 bf16; fused AdaLN fwd+bwd (2 C-ABI calls)",
     "cfg5": "cfg5: batch 4 x 11056 tokens x 3072 bf16, one modulation row per sample; AdaLN then RMSNorm(3072), "
             "forward and backward of the chain (4 C-ABI calls)",
@@ -150,10 +153,14 @@ def build_workload(name, torch, capi, dev):
             x, grad = rnd(712800, 128, dtype=bf), rnd(712800, 128, dtype=bf)
             calls += rms_pair(x, grad, rnd(128, dtype=bf, k=0.02, bias=1.0), tag)[0]
         return calls, 712800 * 128 * 2, 29700, "bf16", x
-    if name == "cfg2-strided":
+    if name in ("cfg2-strided", "cfg2-strided-rope"):
         B, S, H, D = 1, 29700, 24, 128
         mixed = rnd(B, S, H, 3 * D, dtype=bf)
         calls = []
+        rope = name.endswith("-rope")
+        if rope:   # any fp32 tables do for timing; [S, D] as get_1d_rotary_pos_embed(use_real=True) lays them out
+            ang = torch.rand(S, D // 2, device=dev, generator=gen) * 6.28
+            cos, sin = (t.repeat_interleave(2, dim=1).contiguous() for t in (ang.cos(), ang.sin()))
         for i, tag in enumerate(("_q", "_k")):
             view = mixed[..., i * D:(i + 1) * D].transpose(1, 2)          # [B, H, S, D], strides (S*H*3D, 3D, H*3D, 1)
             grad = rnd(B, H, S, D, dtype=bf)
@@ -169,6 +176,15 @@ def build_workload(name, torch, capi, dev):
                    ck(L.tt_rmsnorm_backward_strided(p(dx), p(dw), p(grad), p(view), p(w), p(rstd), B, H, S, xs[0],
                                                     xs[1], xs[2], ds[0], ds[1], ds[2], D, capi.BF16, p(ws), n,
                                                     _LAUNCH_STREAM[0]), "rms bwd strided"))
+            if rope:
+                fwd = (lambda out=out, rstd=rstd, view=view, w=w, xs=xs:
+                       ck(L.tt_rmsnorm_rope_forward_strided(p(out), p(rstd), p(view), p(w), p(cos), p(sin), S, B, H, S,
+                                                            xs[0], xs[1], xs[2], D, EPS, capi.BF16, _LAUNCH_STREAM[0]),
+                          "rms rope fwd strided"))
+                bwd = (lambda dx=dx, dw=dw, grad=grad, view=view, w=w, rstd=rstd, xs=xs, ds=ds, ws=ws, n=n:
+                       ck(L.tt_rmsnorm_rope_backward_strided(p(dx), p(dw), p(grad), p(view), p(w), p(rstd), p(cos), p(sin),
+                                                             S, B, H, S, xs[0], xs[1], xs[2], ds[0], ds[1], ds[2], D,
+                                                             capi.BF16, p(ws), n, _LAUNCH_STREAM[0]), "rms rope bwd strided"))
             calls += [("rmsnorm_forward_strided" + tag, fwd, 2), ("rmsnorm_backward_strided" + tag, bwd, 3)]
         return calls, B * H * S * D * 2, S, "bf16", mixed
     if name == "cfg5":

@@ -9,6 +9,7 @@ kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for 
     python -m teletron_amd.profile_summary workloads --dir rocprof_out     (<dir>/trace_<workload>)
     python -m teletron_amd.profile_summary stream --dir rocprof_out        (<dir>/stream.json, <dir>/stream_stall)
     python -m teletron_amd.profile_summary variants --dir rocprof_out      (<dir>/variant_<name>.json, _sq, _stall)
+    python -m teletron_amd.profile_summary runs --dir rocprof_out          (<dir>/run_<name>_<workload>.json, run_<name>_trace)
 
 The databases are large; run this where they were written and keep only what it writes (--out).
 """
@@ -445,17 +446,75 @@ stream_ceiling.md for what plain streams of the same read/write mix reach.
     print("wrote bench_cfg4_tuning_variants.md")
 
 
+# ------------------------------------------------------------------- run length at the QK-norm site
+
+RUN_VARIANTS = [("run1", 1), ("run3", 3), ("base", 6), ("run12", 12)]
+RUN_WORKLOADS = ["cfg2-strided-rope", "cfg2-strided"]
+
+
+def run_lengths(directory):
+    """bench lines `run_<variant>_<workload>.json`, and kernel traces `run_<variant>_trace` of the rotary
+    site, for the shipped library and builds with other values of TTN_STRIDED_RUN."""
+    digest = kernel_source_digest()
+    rows = ["| groups per run | cfg2-strided-rope ms per step | rotary forward kernel µs | rotary backward kernel µs | "
+            "cfg2-strided ms per step | strided forward / backward µs per call |", "|---|---|---|---|---|---|"]
+    for name, run in RUN_VARIANTS:
+        js = {}
+        for w in RUN_WORKLOADS:
+            f = os.path.join(directory, f"run_{name}_{w}.json")
+            if os.path.exists(f):
+                js[w] = json.loads(open(f).read().strip().splitlines()[-1])
+        if len(js) != len(RUN_WORKLOADS):
+            continue
+        fwd = bwd = float("nan")
+        t = os.path.join(directory, f"run_{name}_trace")
+        if os.path.isdir(t):
+            for r in kernel_stats(t):
+                if "RopeTable" in r["name"]:
+                    if "fwd_kernel" in r["name"]:
+                        fwd = r["avg_us"]
+                    elif "bwd_kernel" in r["name"]:
+                        bwd = r["avg_us"]
+        c = js["cfg2-strided"]["per_call_untimed"]
+        rows.append(f"| {run}{' (shipped)' if name == 'base' else ''} | {js['cfg2-strided-rope']['ms_per_step']:.4f} | {fwd:.1f} | "
+                    f"{bwd:.1f} | {js['cfg2-strided']['ms_per_step']:.4f} | "
+                    f"{c['rmsnorm_forward_strided_q']['median_us']:.1f} / {c['rmsnorm_backward_strided_q']['median_us']:.1f} |")
+    md = f"""# Run length of the strided QK-norm kernels: heads a wavefront takes per table fetch
+
+{BOX}.  Kernel sources digest `{digest}`.  `TTN_STRIDED_RUN` (norm_device.h) is the number of
+consecutive groups -- heads of one token tile -- a wavefront of the strided 128-column kernels takes at a time: the
+rotary kernels fetch the token's cos/sin rows once per run, the backward kernels do the view's index arithmetic once
+per run; the forward kernel without tables always takes single groups.  With 1 every row fetches its own 1 KiB of
+tables (what the kernels did before runs existed).  29 700 tokens x 24 heads x 128, bf16, q and k through the C ABI
+(`cfg2-strided-rope`: the strided norm with the rotation, forward and backward; `cfg2-strided`: without), one box, one
+after the other:
+
+    python -m teletron_amd.build --variant /tmp/lib_run<N>.so --flag=-DTTN_STRIDED_RUN=<N>
+    TELETRON_AMD_LIB=/tmp/lib_run<N>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided-rope
+    TELETRON_AMD_LIB=/tmp/lib_run<N>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided
+    TELETRON_AMD_LIB=/tmp/lib_run<N>.so rocprofv3 --kernel-trace --stats -d {DIR_SHOWN}/run_<name>_trace -o bench -- python3 bench.py --steps 30 --warmup 5 --no-cpu-baseline --workload cfg2-strided-rope
+
+Kernel columns are rocprofv3 averages of `rmsnorm_fwd_kernel<bf16_t, 128, Strided3Rows, RopeTable>` and the matching
+backward kernel.  Written by `python -m teletron_amd.profile_summary runs --dir {DIR_SHOWN}`.
+
+{chr(10).join(rows)}
+"""
+    with open(os.path.join(PROFILES, "qkv_site_run_length_variants.md"), "w") as f:
+        f.write(md)
+    print("wrote qkv_site_run_length_variants.md")
+
+
 def main():
     global PROFILES, DIR_SHOWN
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants"))
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs"))
     ap.add_argument("--dir", default="rocprof_out", help="where rocprofv3 wrote (its -d arguments' parent)")
     ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
     a = ap.parse_args()
     PROFILES = a.out
     DIR_SHOWN = a.dir.rstrip("/")
     os.makedirs(PROFILES, exist_ok=True)
-    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants}[a.what](a.dir)
+    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": run_lengths}[a.what](a.dir)
 
 
 if __name__ == "__main__":
