@@ -26,7 +26,7 @@ from teletron_amd.build import ROOT, kernel_source_digest
 
 PROFILES = os.path.join(ROOT, "profiles")
 DIR_SHOWN = "rocprof_out"   # the --dir argument as typed: what the summaries print in their commands
-OURS = ("rmsnorm_", "adaln_", "stream_copy", "stream_probe", "colreduce")
+OURS = ("rmsnorm_", "adaln_", "stream_copy", "stream_probe", "colreduce", "copy_rows")
 BOX = "MI355X (gfx950, 256 CUs), ROCm 7.2, one GPU"
 
 
@@ -268,6 +268,7 @@ WORKLOAD_INFO = {
     "cfg1": "RMSNorm fwd+bwd, 8192 x 3072 fp32",
     "cfg2": "QK-norm on contiguous q and k, 712 800 rows x 128 bf16",
     "cfg2-strided": "QK-norm on the transposed [B, H, S, D] views into the fused QKV projection, 712 800 rows x 128 bf16",
+    "cfg2-strided-rope": "the same with the rotary embedding applied behind each norm (fp32 tables [29 700, 128])",
     "cfg3": "AdaLN fwd+bwd, 29 700 x 3072 bf16",
     "cfg5": "AdaLN -> RMSNorm chain, 4 x 11 056 x 3072 bf16, one modulation row per sample",
     "w1536-f16": "any-width kernels: RMSNorm + AdaLN fwd+bwd, 237 600 x 1536 fp16",
