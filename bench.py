@@ -288,10 +288,11 @@ def build_workload(name, torch, capi, dev):
 
 
 def stream_ceiling(args, torch, capi, dev):
-    """What the memory system gives plain streams of each read/write mix and access shape (library probe
-    kernels over cfg4-sized tensors), next to two copies not written here: the runtime's device-to-device
-    copy and a PyTorch elementwise copy.  Every figure is back-to-back launches between two events."""
-    L = capi.lib()
+    """What the memory system gives plain streams of each read/write mix and access shape (the probe
+    library's kernels over cfg4-sized tensors), next to two copies not written here: the runtime's
+    device-to-device copy and a PyTorch elementwise copy.  Every figure is back-to-back launches between
+    two events."""
+    from teletron_amd import probe as P
     nbytes = ROWS * COLS * 2
     # two tensors per allocation: the probe's third and fourth read and its second write follow the first
     a = torch.empty(2 * nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -316,11 +317,7 @@ def stream_ceiling(args, torch, capi, dev):
                 "frac_of_peak": round(n_streams * nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
     def probe(reads, writes, per_lane, blocks, through):
-        def fn():
-            st = L.tt_norm_stream_probe(p(d), p(a), p(b), nbytes, reads, writes, per_lane, blocks, through, stream)
-            if st != 0:
-                raise RuntimeError(L.tt_norm_last_error().decode())
-        return timed(fn, reads + writes)
+        return timed(lambda: P.stream(d, a, b, nbytes, reads, writes, per_lane, blocks, through), reads + writes)
 
     rows = []
     for reads, writes in ((1, 0), (2, 0), (0, 1), (1, 1), (2, 1)):
@@ -347,7 +344,7 @@ def stream_ceiling(args, torch, capi, dev):
         "hipMemcpyDtoDAsync": timed(lambda: hip.hipMemcpyDtoDAsync(p(d), p(a), ctypes.c_size_t(nbytes), stream), 2),
         "torch copy_ (bf16)": timed(lambda: d1.view(torch.bfloat16).copy_(a1.view(torch.bfloat16)), 2),
         "torch zero_ (write only)": timed(lambda: d1.view(torch.bfloat16).zero_(), 1),
-        "tt_norm_stream_copy": timed(lambda: capi.stream_copy(d1, a1), 2),
+        "tt_probe_stream_copy": timed(lambda: P.stream_copy(d1, a1), 2),
     }
     best = lambda r_, w_: max((r for r in rows if r["reads"] == r_ and r["writes"] == w_), key=lambda r: r["GB/s"])
     two_one = best(2, 1)
@@ -560,12 +557,13 @@ def main():
     # streaming-copy yardstick (read one tensor, write one tensor) with the same access pattern
     src = a_tensor.reshape(-1)[:tensor_bytes // a_tensor.element_size()]
     dst = torch.empty_like(src)
+    from teletron_amd import probe as P
     for _ in range(3):
-        capi.stream_copy(dst, src)
+        P.stream_copy(dst, src)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(10):
-        capi.stream_copy(dst, src)
+        P.stream_copy(dst, src)
     e1.record()
     torch.cuda.synchronize()
     copy_gbs = 2 * tensor_bytes / (e0.elapsed_time(e1) / 10) / 1e6

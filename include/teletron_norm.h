@@ -41,7 +41,10 @@
 extern "C" {
 #endif
 
-#define TT_NORM_ABI_VERSION 1
+/* 2: adds tt_norm_wide_forms_supported; the gated residual and residual entry points take every row of
+ *    up to 384 16-byte pieces (they took 3072 columns only); the measurement kernels tt_norm_stream_copy
+ *    and tt_norm_stream_probe left this library for libteletron_probe.so (include/teletron_probe.h). */
+#define TT_NORM_ABI_VERSION 2
 
 enum tt_norm_status {
     TT_NORM_OK = 0,
@@ -72,9 +75,16 @@ const char *tt_norm_last_error(void);
 int tt_norm_supported(int64_t cols, int dtype);
 
 /* 1 if (cols, dtype) is one of the tuned shapes (cols 128 or 3072; bf16, fp16 or fp32): the only
- * ones the reference-contract (*_from_out, *_xnorm, *_from_xnorm) and strided entry points
- * take; the gated residual entry points take cols 3072 only. */
+ * ones the reference-contract entry points (*_from_out, *_xnorm, *_from_xnorm) take; the rotary
+ * entry points take cols 128 only.  The strided and sequence-first entry points take whatever
+ * tt_norm_supported accepts. */
 int tt_norm_tuned(int64_t cols, int dtype);
+
+/* 1 if the gated residual and residual entry points (tt_gated_residual_adaln_forward / _backward,
+ * tt_adaln_backward_residual) accept (cols, dtype): 3072 columns in any element type, and every
+ * other supported row of at most 384 16-byte pieces (3072 two-byte / 1536 four-byte columns).
+ * Beyond that those entry points return TT_NORM_EUNSUPPORTED. */
+int tt_norm_wide_forms_supported(int64_t cols, int dtype);
 
 /* ------------------------------------------------------------------ RMSNorm
  * out = round(round(x * rstd) * weight),  rstd = 1/sqrt(mean_c(x^2) + eps)
@@ -218,7 +228,9 @@ int tt_adaln_backward_seq_first(void *dx, void *dscale, void *dshift, const void
  * (tt_adaln_backward_workspace_bytes) exceeds the array return TT_NORM_EWORKSPACE: at 3072
  * columns that is batch > 682; every supported width fits for batch <= 256.  Results are
  * bit-identical to tt_adaln_backward.  All calls on one GPU share that GPU's array: calls that
- * overlap in time on one GPU (different streams or threads) race; on one stream they are safe. */
+ * overlap in time on one GPU (different streams or threads) race; on one stream they are safe.
+ * The array used is the CURRENT device's (hipGetDevice), which must be the device that holds the
+ * tensors: a dx that lives on another device is refused with TT_NORM_EINVAL. */
 #define TT_NORM_STATIC_SCRATCH_BYTES (16u << 20)
 int tt_adaln_backward_static(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
                              const void *scale, const float *mean, const float *rstd,
@@ -235,7 +247,8 @@ int tt_adaln_backward_from_xnorm(void *dx, void *dscale, void *dshift, const voi
 /* tt_adaln_backward for an input that has another consumer (the residual stream continues past the
  * norm, teletron/models/dit/dit_layerspec.py:126-131,152): dres [rows, cols] is the gradient the input
  * receives from that consumer, and dx = round(round(dx of the norm) + dres), the sum autograd would
- * otherwise form in a separate pass.  Same scratch as tt_adaln_backward.  cols must be 3072. */
+ * otherwise form in a separate pass.  Same scratch as tt_adaln_backward.  Shapes:
+ * tt_norm_wide_forms_supported(cols, dtype), else TT_NORM_EUNSUPPORTED. */
 int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *dout, const void *dres,
                                const void *x, const void *scale, const float *mean, const float *rstd,
                                int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
@@ -250,7 +263,8 @@ int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void 
  * norm).  The reference runs these as separate elementwise kernels plus the norm; here
  * one pass reads h and attn and writes h2 and out, and one backward pass produces every
  * gradient.  h, attn, h2, out [batch * rows_per_sample, cols]; gate, scale, shift
- * [batch, cols]; cols must be 3072.
+ * [batch, cols].  Shapes: tt_norm_wide_forms_supported(cols, dtype) -- 3072 columns, or any other
+ * supported row of at most 384 16-byte pieces -- else TT_NORM_EUNSUPPORTED.
  */
 
 int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rstd,
@@ -274,35 +288,16 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                      int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                      void *workspace, size_t workspace_bytes, void *stream);
 
-/* ------------------------------------------------------------- measurement
- * Arms a pair of HIP events (hipEvent_t passed as void*, created by the caller with
- * timing enabled) for the NEXT row kernel launched from this thread: `start` is
- * recorded on that launch's stream immediately before the row kernel and `stop`
- * immediately after it, i.e. before the column reducer of a backward call.  One shot:
- * the pair is disarmed once used.  No counterpart in the reference (which has no
- * instrumentation); it exists so that a benchmark can time exactly the kernel a
- * profiler reports.  Pass NULLs to disarm. */
+/* ------------------------------------------------------------- measurement only
+ * Not part of the operator interface, and no counterpart in the reference (which has no
+ * instrumentation).  Arms a pair of HIP events (hipEvent_t passed as void*, created by the caller
+ * with timing enabled) for the NEXT row kernel launched from this thread: `start` is recorded on that
+ * launch's stream immediately before the row kernel and `stop` immediately after it, i.e. before the
+ * column reducer of a backward call.  One shot: the pair is disarmed once used.  It exists so that a
+ * benchmark can time exactly the kernel a profiler reports; it has to live in this library because
+ * the launch it brackets does.  Pass NULLs to disarm.  The plain streaming kernels the benchmark
+ * compares against are in libteletron_probe.so (teletron_probe.h), not here. */
 int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event);
-
-/*
- * Plain streaming copy of `bytes` (multiple of 16) from src to dst with the
- * same 128-bit access pattern as the kernels: the achievable-bandwidth
- * yardstick the benchmark prints next to each result. */
-int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
-
-/* Measurement only (no counterpart in the reference): a plain stream of `reads` tensors read and `writes`
- * tensors written, `bytes` each, where every wavefront moves one contiguous run of accesses_per_lane KiB
- * per tensor (1, 2 or 6 accesses of 16 bytes per lane; 6 is the shape of a 3072-column two-byte row).
- * Tensors read: a, b, a + bytes, b + bytes (reads 0..4); written: dst, dst + bytes (writes 0..2) -- the
- * allocations must be that long.  Built mixes: up to 2 reads with up to 1 write in every shape; 3+1, 2+2
- * and 4+2 (the mixes of the residual and gated kernels) with 1 and 6 accesses per lane.
- * persistent_blocks = 0 launches one wavefront per run (one-shot grid), otherwise that many workgroups
- * of four wavefronts stride over the runs.  write_through != 0 uses the write-through store of the
- * backward kernels.  The benchmark uses it to print what the memory system gives each read/write mix
- * next to the kernels' own figures.  The event pair armed by tt_norm_profile_next_row_kernel brackets
- * this kernel as well. */
-int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
-                         int accesses_per_lane, int persistent_blocks, int write_through, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,6 +1,8 @@
 """Build recipe for the native parts, all compiled for gfx950 and kept in-tree:
 
   teletron_amd/lib/libteletron_norm.so   HIP kernels + C ABI (include/teletron_norm.h)
+  teletron_amd/lib/libteletron_probe.so  measurement only: plain streaming kernels (include/teletron_probe.h),
+                                         loaded by bench.py and the tests of the probes, never by the operators
   teletron_amd/ext/fused_rmsnorm*.so     PyTorch extension modules with the reference's
   teletron_amd/ext/fused_adaln*.so       module names and torch_launch_* signatures
 
@@ -20,6 +22,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 EXT_DIR = os.path.join(PKG, "ext")
 LIB_PATH = os.path.join(LIB_DIR, "libteletron_norm.so")
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libteletron_probe.so")
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 ARCH = "gfx950"
@@ -75,6 +78,15 @@ def build_kernels(verbose: bool = True, out: str = None, extra_flags=()) -> str:
     return out
 
 
+def build_probe(verbose: bool = True) -> str:
+    """The measurement library: one source, nothing of the operator library linked in."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    log = _run([HIPCC, *HIP_FLAGS, "-shared", "probe.hip", "-o", PROBE_LIB_PATH], cwd=CSRC)
+    if verbose:
+        print("built", os.path.relpath(PROBE_LIB_PATH, ROOT), log.strip())
+    return PROBE_LIB_PATH
+
+
 def ext_path(name: str) -> str:
     suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
     return os.path.join(EXT_DIR, name + suffix)
@@ -109,6 +121,7 @@ def build_extensions(verbose: bool = True):
 
 def build_all(verbose: bool = True):
     build_kernels(verbose)
+    build_probe(verbose)
     build_extensions(verbose)
 
 

@@ -25,11 +25,11 @@ EXPORTS = (
     "tt_rmsnorm_forward", "tt_rmsnorm_backward_workspace_bytes", "tt_rmsnorm_backward",
     "tt_rmsnorm_backward_from_out", "tt_rmsnorm_forward_strided", "tt_rmsnorm_backward_strided",
     "tt_adaln_forward", "tt_adaln_forward_xnorm", "tt_adaln_backward_workspace_bytes",
-    "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_stream_copy",
+    "tt_adaln_backward", "tt_adaln_backward_from_xnorm", "tt_norm_wide_forms_supported",
     "tt_norm_profile_next_row_kernel",
     "tt_gated_residual_adaln_forward", "tt_gated_residual_adaln_backward_workspace_bytes",
     "tt_gated_residual_adaln_backward", "tt_adaln_backward_residual", "tt_adaln_backward_static",
-    "tt_norm_stream_probe", "tt_rmsnorm_rope_forward_strided", "tt_rmsnorm_rope_backward_strided",
+    "tt_rmsnorm_rope_forward_strided", "tt_rmsnorm_rope_backward_strided",
     "tt_adaln_forward_seq_first", "tt_adaln_backward_seq_first", "tt_norm_copy_rows_strided",
 )
 
@@ -56,6 +56,7 @@ def lib() -> ctypes.CDLL:
         L.tt_norm_last_error.restype = ctypes.c_char_p
         L.tt_norm_supported.argtypes = [i64, ci]
         L.tt_norm_tuned.argtypes = [i64, ci]
+        L.tt_norm_wide_forms_supported.argtypes = [i64, ci]
         L.tt_rmsnorm_forward.argtypes = [vp, vp, vp, vp, i64, i64, dbl, ci, vp]
         L.tt_rmsnorm_backward_workspace_bytes.restype = sz
         L.tt_rmsnorm_backward_workspace_bytes.argtypes = [i64, i64, ci]
@@ -79,9 +80,7 @@ def lib() -> ctypes.CDLL:
         L.tt_gated_residual_adaln_backward_workspace_bytes.argtypes = [i64, i64, i64, ci]
         L.tt_gated_residual_adaln_backward.argtypes = [vp] * 13 + [i64, i64, i64, ci, vp, sz, vp]
         L.tt_adaln_backward_residual.argtypes = [vp] * 9 + [i64, i64, i64, ci, vp, sz, vp]
-        L.tt_norm_stream_copy.argtypes = [vp, vp, sz, vp]
         L.tt_norm_copy_rows_strided.argtypes = [vp, vp] + [i64] * 7 + [ci, vp]
-        L.tt_norm_stream_probe.argtypes = [vp, vp, vp, sz, ci, ci, ci, ci, ci, vp]
         L.tt_norm_profile_next_row_kernel.argtypes = [vp, vp]
         _lib = L
     return _lib
@@ -352,10 +351,3 @@ def gated_residual_adaln_backward(dout, dh2, h2, attn, gate, scale, mean, rstd):
                                                   _p(rstd), batch, rows // batch, cols, _dt(h2), _p(ws), n,
                                                   _stream(h2)), "tt_gated_residual_adaln_backward")
     return dh, dattn, dgate, dscale, dshift
-
-
-def stream_copy(dst: torch.Tensor, src: torch.Tensor):
-    _dense_gpu(dst, src)
-    nbytes = src.numel() * src.element_size()
-    with torch.cuda.device(src.device):
-        _check(lib().tt_norm_stream_copy(_p(dst), _p(src), nbytes, _stream(src)), "tt_norm_stream_copy")

@@ -69,6 +69,23 @@
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
+// Backward arithmetic on 2-byte rows taken from the packed pairs (bit 0: gx = rnd(g*t) as one packed
+// dot product per element against masked parameter pairs instead of unpack + multiply; bit 1: the
+// column sums dshift += g and dscale += rnd(g*rnd(xhat)) as packed dot products against (1,0) / (0,1),
+// so g is never unpacked).  A product of two bf16 or fp16 values is exact in fp32, so every rounding
+// point stays where it was.
+#ifndef TTN_BWD_PACKED_MATH
+#define TTN_BWD_PACKED_MATH 3
+#endif
+// Cache-policy bits of the backward kernels' row loads at 3072 columns (sc0 = 1, nt = 2, sc1 = 16) issued as
+// buffer loads over a per-row base in scalar registers; -1 = plain global loads with the non-temporal hint.
+#ifndef TTN_BWD_LOAD_POLICY
+#define TTN_BWD_LOAD_POLICY -1
+#endif
+// Share of the compute units the persistent backward grids at 3072 columns cover, in per cent.
+#ifndef TTN_BWD_GRID_PERCENT
+#define TTN_BWD_GRID_PERCENT 100
+#endif
 
 namespace ttn {
 
@@ -278,12 +295,24 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const int64_t smp = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
 
-    float tv[CHUNKS][VEC];  // t = rnd(1 + scale[sample]), unpacked once
+    constexpr bool kPackedProducts = kHasDot2<T> && (TTN_BWD_PACKED_MATH & 1) != 0;
+    constexpr bool kPackedColumnSums = kHasDot2<T> && (TTN_BWD_PACKED_MATH & 2) != 0;
+    // t = rnd(1 + scale[sample]), resident for the whole kernel: unpacked to fp32, or (packed products) as
+    // the masked pairs (t_lo, 0) and (0, t_hi)
+    using Factor = PairFactor<std::conditional_t<kHasDot2<T>, T, bf16_t>>;  // (unused for 4-byte rows)
+    [[maybe_unused]] const uint32_t one_lo = opaque_const(kOneLo<T>), one_hi = opaque_const(kOneHi<T>);
+    [[maybe_unused]] float tv[kPackedProducts ? 1 : CHUNKS][VEC];
+    [[maybe_unused]] Factor tf[kPackedProducts ? CHUNKS : 1];
     {
         u32x4 tr[CHUNKS];
         load_one_plus_scale<T, C>(tr, scale + smp * C, l);
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k) E::unpack(tr[k], tv[k]);
+        for (int k = 0; k < CHUNKS; ++k) {
+            if constexpr (kPackedProducts)
+                tf[k].set(tr[k]);
+            else
+                E::unpack(tr[k], tv[k]);
+        }
     }
 
     // gate[sample]: unpacked once for 2-byte elements; 4-byte rows have no registers to spare and
@@ -321,11 +350,22 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         b.first = lay.row(smp, grp * RPW) * C;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
+#if TTN_BWD_LOAD_POLICY >= 0
+        if constexpr (LANES == kWaveSize) {
+            const RowReader<TTN_BWD_LOAD_POLICY> rg(g + b.row * C, l * 16), rx(xin + b.row * C, l * 16);
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? rg.get(k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? rx.get(k * LANES) : u32x4{0, 0, 0, 0};
+        } else
+#endif
 #if TTN_BWD_LOAD_RUNS
+        {
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        }
 #else
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
@@ -371,11 +411,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         if constexpr (kDrainStores) wait_memory_ops<0>();
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC];
-            E::unpack(b.g[k], gv);
+            if constexpr (kPackedProducts) {
+                gxp[k] = rounded_products<T>(b.g[k], tf[k]);  // gx materialised in the element type
+            } else {
+                float gv[VEC];
+                E::unpack(b.g[k], gv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) gv[j] *= tv[k][j];
-            gxp[k] = E::pack(gv);  // gx materialised in the element type
+                for (int j = 0; j < VEC; ++j) gv[j] *= tv[k][j];
+                gxp[k] = E::pack(gv);  // gx materialised in the element type
+            }
             if constexpr (kHasDot2<T>) {
                 // s2 accumulates sum_c gx * xin here; turned into sum_c gx * xhat below
 #pragma unroll
@@ -410,15 +454,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         const RowWriter<0> wa(GATED ? da + b.first : nullptr, lane_bytes);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], gx[VEC], xv[VEC], o[VEC], xn[VEC];
-            E::unpack(b.g[k], gv);
+            [[maybe_unused]] float gv[VEC];
+            float gx[VEC], xv[VEC], o[VEC], xn[VEC];
+            if constexpr (!kPackedColumnSums) E::unpack(b.g[k], gv);
             E::unpack(gxp[k], gx);
             E::unpack(b.x[k], xv);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
                 xn[j] = FROM_XNORM ? xv[j] : centred<T>(xv[j], mu, r, nmr);
-                acc[1][k][j] += gv[j];
+                if constexpr (!kPackedColumnSums) acc[1][k][j] += gv[j];
             }
             if constexpr (GATED) {
                 float ev[VEC], av[VEC], dav[VEC];
@@ -464,12 +509,28 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 }
                 if (b.ok) wd.put(k * LANES, E::pack(o));
             }
-            if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
+            if constexpr (kPackedColumnSums) {
+                Factor nf;  // the normalised row in the element type
+                if constexpr (FROM_XNORM)
+                    nf.set(b.x[k]);
+                else
+                    nf.set_rounded(xn);
+                const u32x4 pp = rounded_products<T>(b.g[k], nf);  // g*xn in the element type, then summed
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
-            E::round(xn);  // g*xn materialised in the element type before the column sum
+                for (int i = 0; i < 4; ++i) {
+                    acc[0][k][2 * i] = dot2<T>(pp[i], one_lo, acc[0][k][2 * i]);
+                    acc[0][k][2 * i + 1] = dot2<T>(pp[i], one_hi, acc[0][k][2 * i + 1]);
+                    acc[1][k][2 * i] = dot2<T>(b.g[k][i], one_lo, acc[1][k][2 * i]);
+                    acc[1][k][2 * i + 1] = dot2<T>(b.g[k][i], one_hi, acc[1][k][2 * i + 1]);
+                }
+            } else {
+                if constexpr (!FROM_XNORM) E::round(xn);  // the normalised row in the element type
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[0][k][j] += xn[j];
+                for (int j = 0; j < VEC; ++j) xn[j] *= gv[j];
+                E::round(xn);  // g*xn materialised in the element type before the column sum
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[0][k][j] += xn[j];
+            }
         }
     };
 
@@ -538,7 +599,8 @@ static int adaln_forward_t(void *out, void *xnorm, float *mean, float *rstd, con
 
 template <typename T, int C>
 static RowPlan adaln_backward_plan(int64_t batch, int64_t rows_per_sample, int cus) {
-    return make_row_plan(batch, rows_per_sample, RowGeom<T, C>::RPW, AdalnTune<T, C>::kBwdBlocksPerCu, cus);
+    const int share = C >= 1024 ? (cus * TTN_BWD_GRID_PERCENT + 99) / 100 : cus;
+    return make_row_plan(batch, rows_per_sample, RowGeom<T, C>::RPW, AdalnTune<T, C>::kBwdBlocksPerCu, share);
 }
 
 template <typename T, int C, bool FROM_XNORM, bool GATED = false, bool RES = false>
@@ -788,18 +850,32 @@ int tt_adaln_backward_static(void *dx, void *dscale, void *dshift, const void *d
     void *ws = nullptr;
     st = static_scratch_address(&ws);
     if (st != TT_NORM_OK) return st;
+    if (rows_per_sample > 0) {
+        // the array belongs to the current device; tensors on another one would be paired with the wrong copy
+        int dev = -1;
+        hipPointerAttribute_t attr;
+        if (hipGetDevice(&dev) != hipSuccess || hipPointerGetAttributes(&attr, dx) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(TT_NORM_EINVAL, "tt_adaln_backward_static: dx is not a device pointer the runtime knows");
+        }
+        if (attr.device != dev)
+            return fail(TT_NORM_EINVAL, "tt_adaln_backward_static: dx lives on device %d, the current device is %d",
+                        attr.device, dev);
+    }
     // every partial row the reducer reads is written in full by the row kernel of the same call:
     // nothing in the array has to start at zero
     return tt_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols, dtype, ws,
                              kStaticScratchBytes, stream);
 }
 
-/* ---- gated residual + AdaLN (3072 columns) ---- */
+/* ---- gated residual + AdaLN (3072 columns, or any row of up to 384 16-byte pieces) ---- */
 
 int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h,
                                     const void *attn, const void *gate, const void *scale,
                                     const void *shift, int64_t batch, int64_t rows_per_sample,
                                     int64_t cols, double eps, int dtype, void *stream) {
+    if (tt_norm_supported(cols, dtype) && !tt_norm_wide_forms_supported(cols, dtype))
+        return wide_form_unsupported("tt_gated_residual_adaln_forward", cols);
     int st = check_adaln_args("tt_gated_residual_adaln_forward", batch, rows_per_sample, cols, dtype,
                               {h2, out, h, attn, gate, scale, shift});
     if (st != TT_NORM_OK) return st;
@@ -821,7 +897,7 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
 
 size_t tt_gated_residual_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols,
                                                         int dtype) {
-    if (cols != 3072 && !anywidth_wide_forms_supported(cols, dtype)) return 0;
+    if (!tt_norm_wide_forms_supported(cols, dtype)) return 0;
     // three sets of column sums (dscale, dshift, dgate) instead of two
     return tt_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype) / 2 * 3;
 }
@@ -832,6 +908,8 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                      const float *rstd, int64_t batch, int64_t rows_per_sample,
                                      int64_t cols, int dtype, void *workspace, size_t workspace_bytes,
                                      void *stream) {
+    if (tt_norm_supported(cols, dtype) && !tt_norm_wide_forms_supported(cols, dtype))
+        return wide_form_unsupported("tt_gated_residual_adaln_backward", cols);
     int st = check_adaln_args("tt_gated_residual_adaln_backward", batch, rows_per_sample, cols, dtype,
                               {dh, dattn, dout, h2, attn, gate, scale});
     if (st != TT_NORM_OK) return st;
@@ -856,12 +934,14 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
                                                       workspace, workspace_bytes, a, dgate, gp);
 }
 
-/* ---- AdaLN backward with the input's other gradient added in (3072 columns) ---- */
+/* ---- AdaLN backward with the input's other gradient added in (same shapes as the gated form) ---- */
 
 int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *dout, const void *dres,
                                const void *x, const void *scale, const float *mean, const float *rstd,
                                int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,
                                void *workspace, size_t workspace_bytes, void *stream) {
+    if (tt_norm_supported(cols, dtype) && !tt_norm_wide_forms_supported(cols, dtype))
+        return wide_form_unsupported("tt_adaln_backward_residual", cols);
     int st = check_adaln_args("tt_adaln_backward_residual", batch, rows_per_sample, cols, dtype,
                               {dx, dout, dres, x, scale});
     if (st != TT_NORM_OK) return st;

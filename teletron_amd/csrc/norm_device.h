@@ -64,6 +64,24 @@ inline constexpr bool kHasDot2 = sizeof(T) == 2;
 template <typename T>
 inline constexpr uint32_t kOnesPair = kIsBf16<T> ? 0x3F803F80u : 0x3C003C00u;
 
+// (1, 0) and (0, 1) as pairs of T: a packed dot product against one of them adds one half of a pair
+// to an fp32 accumulator, and a pair with one half cleared turns the packed dot product into the
+// exact fp32 product of the other halves -- "unpack and multiply" / "unpack and add" in one
+// instruction per element instead of two.
+template <typename T>
+inline constexpr uint32_t kOneLo = kIsBf16<T> ? 0x00003F80u : 0x00003C00u;
+template <typename T>
+inline constexpr uint32_t kOneHi = kIsBf16<T> ? 0x3F800000u : 0x3C000000u;
+
+// A 32-bit constant handed to the compiler in a scalar register whose value it cannot see.  Needed for
+// pair constants that are operands of the packed bf16 dot product: the compiler encodes the pair
+// (1.0, 0) as the inline operand 1.0, which the hardware reads as the fp32 number 1.0 -- the pair
+// (0, 1.0) -- so both halves of a column-sum update would add the upper element.
+__device__ __forceinline__ uint32_t opaque_const(uint32_t v) {
+    asm("" : "+s"(v));
+    return v;
+}
+
 // acc + a.lo*b.lo + a.hi*b.hi over one dword of two elements each (v_dot2c_f32_bf16 /
 // v_dot2_f32_f16): products of bf16 or fp16 pairs are exact in fp32, so this is a row
 // reduction step taken straight from the packed registers, with no unpacking.
@@ -89,6 +107,7 @@ struct Elem<bf16_t> {
             v[2 * i + 1] = as_f32(r[i] & 0xffff0000u);
         }
     }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
     static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
         u32x4 r;
 #pragma unroll
@@ -116,21 +135,21 @@ struct Elem<f16_t> {
             v[2 * i + 1] = (float)h[1];
         }
     }
+    // The value is an fp32 number before it is converted, as in the eager formulas (an fp32 op, then
+    // .to(half)).  Left to itself the compiler folds the producing multiply into a mixed-precision
+    // instruction in some kernels and not in others, and one element in ten thousand then differs
+    // by an ulp from kernel to kernel.
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        asm("" : "+v"(lo), "+v"(hi));
+        f16x2_t h;
+        h[0] = (_Float16)lo;
+        h[1] = (_Float16)hi;
+        return __builtin_bit_cast(uint32_t, h);
+    }
     static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
         u32x4 r;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // The value is an fp32 number before it is converted, as in the eager formulas (an fp32 op, then
-            // .to(half)).  Left to itself the compiler folds the producing multiply into a mixed-precision
-            // instruction in some kernels and not in others, and one element in ten thousand then differs
-            // by an ulp from kernel to kernel.
-            float lo = v[2 * i], hi = v[2 * i + 1];
-            asm("" : "+v"(lo), "+v"(hi));
-            f16x2_t h;
-            h[0] = (_Float16)lo;
-            h[1] = (_Float16)hi;
-            r[i] = __builtin_bit_cast(uint32_t, h);
-        }
+        for (int i = 0; i < 4; ++i) r[i] = pack2(v[2 * i], v[2 * i + 1]);
         return r;
     }
     static __device__ __forceinline__ void round(float (&v)[8]) {
@@ -154,6 +173,87 @@ struct Elem<float> {
     }
     static __device__ __forceinline__ void round(float (&)[4]) {}
 };
+
+// ---- rounded products straight from packed pairs ------------------------------------
+// rnd(a*b) for the eight elements of a 16-byte piece, both factors 2-byte values: the product of two
+// bf16 or fp16 values is exact in fp32, so rounding it once to the element type is what the eager
+// formulas do when they multiply two tensors of that type.
+//   fp16: the packed half multiply (v_pk_mul_f16) is that operation, one instruction per pair.
+//   bf16: there is no packed bf16 multiply; the packed dot product  a.lo*b.lo + a.hi*b.hi + 0  against a
+//     pair with one half cleared is the exact product of the other halves: one instruction per
+//     element where unpacking and multiplying takes two.  The second factor is therefore held as the
+//     two masked pairs (b.lo, 0) and (0, b.hi).
+// PairFactor<T> is the second factor in the form its type wants; it can be set from packed pairs or
+// from eight fp32 values that are rounded to the element type on the way.
+template <typename T>
+struct PairFactor;
+
+template <>
+struct PairFactor<bf16_t> {
+    uint32_t lo[4], hi[4];
+    __device__ __forceinline__ void set(const u32x4 &p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo[i] = p[i] & 0x0000ffffu;
+            hi[i] = p[i] & 0xffff0000u;
+        }
+    }
+    __device__ __forceinline__ void set_rounded(const float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // (rnd(v), 0) and (0, rnd(v)) in one conversion each; written out because the compiler builds
+            // the pair with a constant half from a conversion plus a byte permute
+            asm("v_cvt_pk_bf16_f32 %0, %1, 0" : "=v"(lo[i]) : "v"(v[2 * i]));
+            asm("v_cvt_pk_bf16_f32 %0, 0, %1" : "=v"(hi[i]) : "v"(v[2 * i + 1]));
+        }
+    }
+};
+
+template <>
+struct PairFactor<f16_t> {
+    u32x4 p;
+    __device__ __forceinline__ void set(const u32x4 &v) { p = v; }
+    __device__ __forceinline__ void set_rounded(const float (&v)[8]) { p = Elem<f16_t>::pack(v); }
+};
+
+template <typename T>
+__device__ __forceinline__ u32x4 rounded_products(const u32x4 &a, const PairFactor<T> &b);
+
+template <>
+__device__ __forceinline__ u32x4 rounded_products<f16_t>(const u32x4 &a, const PairFactor<f16_t> &b) {
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        r[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2_t, (uint32_t)a[i]) *
+                                                __builtin_bit_cast(f16x2_t, (uint32_t)b.p[i]));
+    return r;
+}
+
+// Written as one block of instructions because the compiler only knows the accumulating form of the
+// bf16 dot product (it clears a register first: two instructions per product again), and because a
+// register written by a dot-product instruction may be read by another kind of instruction only three
+// or more instructions later: the block keeps that distance itself (each conversion reads products
+// issued at least three instructions before it), and what leaves the block was written by conversions.
+template <>
+__device__ __forceinline__ u32x4 rounded_products<bf16_t>(const u32x4 &a, const PairFactor<bf16_t> &b) {
+    uint32_t r0, r1, r2, r3, q0, q1, q2, q3;
+    asm("v_dot2_f32_bf16 %0, %8, %12, 0\n\t"
+        "v_dot2_f32_bf16 %4, %8, %16, 0\n\t"
+        "v_dot2_f32_bf16 %1, %9, %13, 0\n\t"
+        "v_dot2_f32_bf16 %5, %9, %17, 0\n\t"
+        "v_dot2_f32_bf16 %2, %10, %14, 0\n\t"
+        "v_dot2_f32_bf16 %6, %10, %18, 0\n\t"
+        "v_dot2_f32_bf16 %3, %11, %15, 0\n\t"
+        "v_dot2_f32_bf16 %7, %11, %19, 0\n\t"
+        "v_cvt_pk_bf16_f32 %0, %0, %4\n\t"
+        "v_cvt_pk_bf16_f32 %1, %1, %5\n\t"
+        "v_cvt_pk_bf16_f32 %2, %2, %6\n\t"
+        "v_cvt_pk_bf16_f32 %3, %3, %7"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3)
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b.lo[0]), "v"(b.lo[1]), "v"(b.lo[2]), "v"(b.lo[3]),
+          "v"(b.hi[0]), "v"(b.hi[1]), "v"(b.hi[2]), "v"(b.hi[3]));
+    return u32x4{r0, r1, r2, r3};
+}
 
 template <typename T, int C>
 struct RowGeom {
@@ -209,6 +309,25 @@ struct RowWriter<1> {
     }
     __device__ __forceinline__ void put(int piece, const u32x4 &v) const {
         __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, piece * 16, kSc1Nt);
+    }
+};
+
+// Where a wavefront reads one row from when the row's address is wave-uniform (one row per wavefront):
+// the base in scalar registers, as RowWriter<1>, so that the load can carry any cache-policy bits
+// (sc0 = 1, nt = 2, sc1 = 16); get(piece) loads the lane's 16 bytes at 16-byte piece `piece`.
+template <int POLICY>
+struct RowReader {
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t off;
+    __device__ __forceinline__ RowReader(const void *wave_base, uint32_t lane_bytes) : off(lane_bytes) {
+        const uint64_t a = reinterpret_cast<uint64_t>(wave_base);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(((uint64_t)hi << 32) | lo), 0, 0xffffffffu,
+                                                 RowWriter<1>::kRawDwords);
+    }
+    __device__ __forceinline__ u32x4 get(int piece) const {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, piece * 16, POLICY);
     }
 };
 

@@ -1,6 +1,5 @@
-// Status handling, device facts, launch geometry, the fixed-order column
-// reducer (stage 2 of every parameter-gradient reduction) and the streaming
-// copy used as the bandwidth yardstick.
+// Status handling, device facts, launch geometry and the fixed-order column
+// reducer (stage 2 of every parameter-gradient reduction).
 #include "norm_host.h"
 
 #include <atomic>
@@ -153,84 +152,6 @@ int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, i
     return check_launch("column reducer launch");
 }
 
-// ---- streaming copy ----------------------------------------------------------
-// The fastest plain copy found on this part, used as the yardstick next to the
-// kernels: one-shot grid, every wavefront copies one contiguous 6 KiB run (six
-// 16-byte accesses per lane, the shape of a 3072-wide bf16 row) and exits.
-__global__ __launch_bounds__(kRowThreads) void stream_copy_kernel(u32x4 *__restrict__ dst,
-                                                                  const u32x4 *__restrict__ src, size_t n16) {
-    constexpr int kDepth = 6;
-    const int lane = threadIdx.x & 63;
-    const size_t wave = (size_t)blockIdx.x * kRowWaves + wave_id_in_block();
-    const size_t base = wave * (kDepth * kWaveSize) + lane;
-    u32x4 v[kDepth];
-#pragma unroll
-    for (int k = 0; k < kDepth; ++k) {
-        const size_t i = base + (size_t)k * kWaveSize;
-        if (i < n16) v[k] = load16_stream(src + i);
-    }
-#pragma unroll
-    for (int k = 0; k < kDepth; ++k) {
-        const size_t i = base + (size_t)k * kWaveSize;
-        if (i < n16) store16_stream(dst + i, v[k]);
-    }
-}
-
-// ---- streaming probe -----------------------------------------------------------
-// Plain streams with the access shapes the row kernels can choose from, for measuring what this
-// memory system gives each read/write mix: NR tensors read (0..4), NW written (0..2);
-// every wavefront moves one contiguous run of D KiB per tensor (D 16-byte accesses per lane; 6 is
-// a 3072-column two-byte row) and either exits (one-shot grid) or strides on (persistent grid).
-// Loads carry the non-temporal hint; THROUGH picks the store (see RowWriter).
-struct ProbeTensors {
-    const u32x4 *read[4];
-    u32x4 *write[2];
-};
-
-template <int NR, int NW, int D, int THROUGH>
-__global__ __launch_bounds__(kRowThreads) void stream_probe_kernel(const ProbeTensors t, int64_t runs,
-                                                                   u32x4 *__restrict__ sink) {
-    const int lane = threadIdx.x & 63;
-    u32x4 keep{0, 0, 0, 0};
-    const int64_t stride = (int64_t)gridDim.x * kRowWaves;
-    for (int64_t run = (int64_t)blockIdx.x * kRowWaves + wave_id_in_block(); run < runs; run += stride) {
-        const int64_t at = run * (D * kWaveSize);
-        u32x4 v[NR > 0 ? NR : 1][D];
-        if constexpr (NR == 0) {
-#pragma unroll
-            for (int k = 0; k < D; ++k) v[0][k] = u32x4{(uint32_t)run, 1, 2, 3};
-        }
-#pragma unroll
-        for (int i = 0; i < NR; ++i)
-#pragma unroll
-            for (int k = 0; k < D; ++k) v[i][k] = load16_stream(t.read[i] + at + lane + k * kWaveSize);
-#pragma unroll
-        for (int i = 1; i < NR; ++i)
-#pragma unroll
-            for (int k = 0; k < D; ++k) v[0][k] += v[i][k];
-        if constexpr (NW >= 1) {
-#pragma unroll
-            for (int j = 0; j < NW; ++j) {
-                const RowWriter<THROUGH> wr(t.write[j] + at, lane * 16);
-#pragma unroll
-                for (int k = 0; k < D; ++k) wr.put(k * kWaveSize, v[0][k] + (uint32_t)j);
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < D; ++k) keep += v[0][k];
-        }
-    }
-    // read-only probes: keep the loads alive without ever storing
-    if (NW == 0 && keep[0] == 0x12345678u && keep[1] == 0x9abcdef0u && keep[2] == 0x0fedcba9u) *sink = keep;
-}
-
-template <int NR, int NW, int D, int THROUGH>
-static int launch_stream_probe(const ProbeTensors &t, int64_t runs, int64_t blocks, hipStream_t stream) {
-    RowKernelProfile prof(stream);
-    stream_probe_kernel<NR, NW, D, THROUGH><<<dim3((unsigned)blocks), dim3(kRowThreads), 0, stream>>>(t, runs, t.write[0]);
-    return TT_NORM_OK;
-}
-
 }  // namespace ttn
 
 using namespace ttn;
@@ -259,67 +180,17 @@ int tt_norm_supported(int64_t cols, int dtype) {
 
 int tt_norm_tuned(int64_t cols, int dtype) { return tuned_shape(cols, dtype) ? 1 : 0; }
 
+int tt_norm_wide_forms_supported(int64_t cols, int dtype) {
+    if (dtype != TT_NORM_BF16 && dtype != TT_NORM_F16 && dtype != TT_NORM_F32) return 0;
+    return (cols == 3072 || anywidth_wide_forms_supported(cols, dtype)) ? 1 : 0;
+}
+
 int tt_norm_profile_next_row_kernel(void *start_event, void *stop_event) {
     if ((start_event == nullptr) != (stop_event == nullptr))
         return fail(TT_NORM_EINVAL, "profile_next_row_kernel: pass both events or neither");
     g_profile_start = (hipEvent_t)start_event;
     g_profile_stop = (hipEvent_t)stop_event;
     return TT_NORM_OK;
-}
-
-int tt_norm_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
-    if (!dst || !src) return fail(TT_NORM_EINVAL, "stream_copy: null pointer");
-    if (bytes % 16) return fail(TT_NORM_EINVAL, "stream_copy: bytes (%zu) not a multiple of 16", bytes);
-    if (!aligned16(dst) || !aligned16(src)) return fail(TT_NORM_EALIGN, "stream_copy: unaligned pointer");
-    if (bytes == 0) return TT_NORM_OK;
-    const size_t n16 = bytes / 16;
-    const size_t per_block = (size_t)kRowWaves * 6 * kWaveSize;
-    const size_t blocks = (n16 + per_block - 1) / per_block;
-    if (blocks > 0x7fffffffULL) return fail(TT_NORM_EINVAL, "stream_copy: %zu bytes is too large for one launch", bytes);
-    stream_copy_kernel<<<dim3((unsigned)blocks), dim3(kRowThreads), 0, (hipStream_t)stream>>>(
-        (u32x4 *)dst, (const u32x4 *)src, n16);
-    return check_launch("stream copy launch");
-}
-
-int tt_norm_stream_probe(void *dst, const void *a, const void *b, size_t bytes, int reads, int writes,
-                         int accesses_per_lane, int persistent_blocks, int write_through, void *stream) {
-    if (reads < 0 || reads > 4 || writes < 0 || writes > 2 || reads + writes == 0)
-        return fail(TT_NORM_EINVAL, "stream_probe: reads=%d (0..4) writes=%d (0..2), at least one stream", reads, writes);
-    if (accesses_per_lane != 1 && accesses_per_lane != 2 && accesses_per_lane != 6)
-        return fail(TT_NORM_EUNSUPPORTED, "stream_probe: accesses_per_lane=%d (built for 1, 2 and 6)", accesses_per_lane);
-    if (persistent_blocks < 0) return fail(TT_NORM_EINVAL, "stream_probe: persistent_blocks=%d", persistent_blocks);
-    const size_t run_bytes = (size_t)accesses_per_lane * kWaveSize * 16;
-    if (bytes == 0 || bytes % run_bytes)
-        return fail(TT_NORM_EINVAL, "stream_probe: bytes (%zu) must be a positive multiple of %zu", bytes, run_bytes);
-    if (!dst || (reads >= 1 && !a) || (reads >= 2 && !b)) return fail(TT_NORM_EINVAL, "stream_probe: null pointer");
-    if (!aligned16(dst) || !aligned16(a) || !aligned16(b)) return fail(TT_NORM_EALIGN, "stream_probe: unaligned pointer");
-    const int64_t runs = (int64_t)(bytes / run_bytes);
-    const int64_t blocks = persistent_blocks ? persistent_blocks : (runs + kRowWaves - 1) / kRowWaves;
-    if (blocks > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "stream_probe: grid too large");
-    const hipStream_t s = (hipStream_t)stream;
-    const int through = (write_through && writes) ? 1 : 0;
-    // tensors 3 and 4 read, and the second one written, follow the first ones in the same allocations
-    const char *ca = (const char *)a, *cb = (const char *)b;
-    char *cd = (char *)dst;
-    const ProbeTensors t{{(const u32x4 *)ca, (const u32x4 *)cb, (const u32x4 *)(ca + bytes), (const u32x4 *)(cb + bytes)},
-                         {(u32x4 *)cd, (u32x4 *)(cd + bytes)}};
-#define TTN_PROBE(NR, NW, D, TH)                                                          \
-    if (reads == NR && writes == NW && accesses_per_lane == D && through == TH) {         \
-        launch_stream_probe<NR, NW, D, TH>(t, runs, blocks, s);                           \
-        return check_launch("stream probe launch");                                       \
-    }
-#define TTN_PROBE_D(NR, NW, TH) TTN_PROBE(NR, NW, 1, TH) TTN_PROBE(NR, NW, 2, TH) TTN_PROBE(NR, NW, 6, TH)
-    TTN_PROBE_D(1, 0, 0) TTN_PROBE_D(2, 0, 0)
-    TTN_PROBE_D(0, 1, 0) TTN_PROBE_D(1, 1, 0) TTN_PROBE_D(2, 1, 0)
-    TTN_PROBE_D(0, 1, 1) TTN_PROBE_D(1, 1, 1) TTN_PROBE_D(2, 1, 1)
-#undef TTN_PROBE_D
-    // the mixes of the gated residual kernels (forward 2 reads + 2 writes, backward 4 + 2) and of the
-    // backward with a residual gradient (3 + 1), in the one-row and the 1 KiB shapes
-#define TTN_PROBE_W(NR, NW) TTN_PROBE(NR, NW, 1, 0) TTN_PROBE(NR, NW, 6, 0) TTN_PROBE(NR, NW, 1, 1) TTN_PROBE(NR, NW, 6, 1)
-    TTN_PROBE_W(3, 1) TTN_PROBE_W(2, 2) TTN_PROBE_W(4, 2)
-#undef TTN_PROBE_W
-#undef TTN_PROBE
-    return fail(TT_NORM_EUNSUPPORTED, "stream_probe: no kernel for this combination");
 }
 
 }  // extern "C"

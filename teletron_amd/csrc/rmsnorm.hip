@@ -41,6 +41,22 @@
 #ifndef TTN_BWD_WAVES_PER_SIMD
 #define TTN_BWD_WAVES_PER_SIMD 1
 #endif
+// Backward arithmetic on 2-byte rows taken from the packed pairs (bit 0: gy = rnd(g*w) as one packed
+// dot product per element against masked weight pairs instead of unpack + multiply; bit 1: the column
+// sum dw += rnd(g*rnd(x*r)) as packed dot products, so g is never unpacked).  A product of two bf16 or
+// fp16 values is exact in fp32, so every rounding point stays where it was.
+#ifndef TTN_BWD_PACKED_MATH
+#define TTN_BWD_PACKED_MATH 3
+#endif
+// Cache-policy bits of the backward kernels' row loads at 3072 columns (sc0 = 1, nt = 2, sc1 = 16) issued as
+// buffer loads over a per-row base in scalar registers; -1 = plain global loads with the non-temporal hint.
+#ifndef TTN_BWD_LOAD_POLICY
+#define TTN_BWD_LOAD_POLICY -1
+#endif
+// Share of the compute units the persistent backward grids at 3072 columns cover, in per cent.
+#ifndef TTN_BWD_GRID_PERCENT
+#define TTN_BWD_GRID_PERCENT 100
+#endif
 // Stores of dx / out: 1 = write-through at device scope (RowWriter<1>), 0 = plain streaming store.
 // Backward (2 reads + 1 write): 367 -> 353 us with write-through.  Forward (1 read + 1 write): the same
 // either way at 3072 columns (one-shot grid), 62.6 -> 61.4 us at 128 columns (persistent grid).
@@ -266,11 +282,20 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     const int l = lane % LANES;
     const int wave = wave_id_in_block();
 
-    float wv[CHUNKS][VEC];                     // weight, unpacked once
-    [[maybe_unused]] float winv[CHUNKS][VEC];  // 1/weight for the saved-output variant
+    constexpr bool kPackedProducts = kHasDot2<T> && (TTN_BWD_PACKED_MATH & 1) != 0;
+    constexpr bool kPackedColumnSums = kPackedDot && (TTN_BWD_PACKED_MATH & 2) != 0;
+    // the weight, resident for the whole kernel: unpacked to fp32, or (packed products) as the masked
+    // pairs (w_lo, 0) and (0, w_hi)
+    using Factor = PairFactor<std::conditional_t<kHasDot2<T>, T, bf16_t>>;  // (unused for 4-byte rows)
+    [[maybe_unused]] const uint32_t one_lo = opaque_const(kOneLo<T>), one_hi = opaque_const(kOneHi<T>);
+    [[maybe_unused]] float wv[(kPackedProducts && !FROM_OUT) ? 1 : CHUNKS][VEC];
+    [[maybe_unused]] Factor wf[kPackedProducts ? CHUNKS : 1];
+    [[maybe_unused]] float winv[FROM_OUT ? CHUNKS : 1][VEC];  // 1/weight for the saved-output variant
 #pragma unroll
     for (int k = 0; k < CHUNKS; ++k) {
-        E::unpack(load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l), wv[k]);
+        const u32x4 wr = load16(reinterpret_cast<const u32x4 *>(w) + k * LANES + l);
+        if constexpr (kPackedProducts) wf[k].set(wr);
+        if constexpr (!kPackedProducts || FROM_OUT) E::unpack(wr, wv[k]);
         if constexpr (FROM_OUT) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) winv[k][j] = __builtin_amdgcn_rcpf(wv[k][j]);
@@ -331,11 +356,22 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         b.dlane = (uint32_t)((at.doff - b.doff0) * (int64_t)sizeof(T)) + l * 16;
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + at.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + at.xoff) + l;
+#if TTN_BWD_LOAD_POLICY >= 0
+        if constexpr (LANES == kWaveSize) {
+            const RowReader<TTN_BWD_LOAD_POLICY> rg(g + at.row * C, l * 16), rx(xin + at.xoff, l * 16);
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? rg.get(k * LANES) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? rx.get(k * LANES) : u32x4{0, 0, 0, 0};
+        } else
+#endif
 #if TTN_BWD_LOAD_RUNS
+        {
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) b.g[k] = b.ok ? load16_stream(pg + k * LANES) : u32x4{0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) b.x[k] = b.ok ? load16_stream(px + k * LANES) : u32x4{0, 0, 0, 0};
+        }
 #else
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
@@ -370,11 +406,15 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         if constexpr (kDrainStores) wait_memory_ops<0>();
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC];
-            E::unpack(b.g[k], gv);
+            if constexpr (kPackedProducts) {
+                gyp[k] = rounded_products<T>(b.g[k], wf[k]);  // gy materialised in the element type
+            } else {
+                float gv[VEC];
+                E::unpack(b.g[k], gv);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) gv[j] *= wv[k][j];
-            gyp[k] = E::pack(gv);  // gy materialised in the element type
+                for (int j = 0; j < VEC; ++j) gv[j] *= wv[k][j];
+                gyp[k] = E::pack(gv);  // gy materialised in the element type
+            }
             if constexpr (kPackedDot) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) dot = dot2<T>(gyp[k][i], b.x[k][i], dot);
@@ -394,8 +434,9 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         const RowWriter<TTN_RMS_BWD_STORE> wd(dx + b.doff0, b.dlane);
 #pragma unroll
         for (int k = 0; k < CHUNKS; ++k) {
-            float gv[VEC], gy[VEC], xv[VEC], o[VEC], y[VEC];
-            E::unpack(b.g[k], gv);
+            [[maybe_unused]] float gv[VEC];
+            float gy[VEC], xv[VEC], o[VEC], y[VEC];
+            if constexpr (!kPackedColumnSums) E::unpack(b.g[k], gv);
             E::unpack(gyp[k], gy);
             E::unpack(b.x[k], xv);
 #pragma unroll
@@ -405,12 +446,23 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
                 y[j] = FROM_OUT ? xs : xs * r;
             }
             if (b.ok) wd.put(k * LANES, E::pack(o));
-            E::round(y);  // y = normalised row in the element type
+            if constexpr (kPackedColumnSums) {
+                Factor yf;  // y = the normalised row in the element type
+                yf.set_rounded(y);
+                const u32x4 pp = rounded_products<T>(b.g[k], yf);  // g*y in the element type, then summed
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
-            E::round(y);  // g*y materialised in the element type before the column sum
+                for (int i = 0; i < 4; ++i) {
+                    acc[0][k][2 * i] = dot2<T>(pp[i], one_lo, acc[0][k][2 * i]);
+                    acc[0][k][2 * i + 1] = dot2<T>(pp[i], one_hi, acc[0][k][2 * i + 1]);
+                }
+            } else {
+                E::round(y);  // y = normalised row in the element type
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[0][k][j] += y[j];
+                for (int j = 0; j < VEC; ++j) y[j] *= gv[j];
+                E::round(y);  // g*y materialised in the element type before the column sum
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[0][k][j] += y[j];
+            }
         }
     };
 
@@ -491,7 +543,8 @@ static int rmsnorm_forward_t(void *out, float *rstd, const void *x, const void *
 // also for strided views: a persistent grid covers any traversal.
 template <typename T, int C>
 static RowPlan rmsnorm_backward_plan(int64_t rows, int cus) {
-    return make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kBwdBlocksPerCu, cus);
+    const int share = C >= 1024 ? (cus * TTN_BWD_GRID_PERCENT + 99) / 100 : cus;
+    return make_row_plan(1, rows, RowGeom<T, C>::RPW, RmsTune<T, C>::kBwdBlocksPerCu, share);
 }
 
 template <typename T, int C, bool FROM_OUT, typename Map, typename Rope = NoRope>

@@ -13,8 +13,8 @@ from oracle import norm_oracle as O
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "teletron_norm.h")).read()
+def _declared_functions(header="teletron_norm.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tt_\w+)\s*\(", text)))
 
@@ -27,7 +27,7 @@ def test_c_abi_exports_every_declared_symbol():
     for n in names:
         assert hasattr(L, n), f"{n} declared in teletron_norm.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert L.tt_norm_abi_version() == 1
+    assert L.tt_norm_abi_version() == 2
     assert L.tt_norm_status_string(0) == b"ok"
     assert L.tt_norm_status_string(4).startswith(b"workspace")
     assert L.tt_norm_supported(3072, capi.BF16) == 1 and L.tt_norm_supported(128, capi.F32) == 1
@@ -52,7 +52,54 @@ def test_c_abi_argument_errors_need_no_gpu():
     assert b"cols=1004" in L.tt_norm_last_error()
     assert L.tt_rmsnorm_forward(None, None, None, None, 4, 1000, 1e-6, 0, None) == 1      # supported; null pointers
     assert L.tt_adaln_forward(None, None, None, None, None, None, 0, 4, 3072, 1e-6, 0, None) == 1
-    assert L.tt_norm_stream_copy(None, None, 32, None) == 1
+
+
+def test_probe_library_is_separate_and_exports_its_header():
+    """The measurement kernels live in a library of their own: its header's symbols are exported there, none of
+    them by the operator library, and its argument checks answer before anything is launched."""
+    from teletron_amd import capi, probe
+    P, L = probe.lib(), capi.lib()
+    names = _declared_functions("teletron_probe.h")
+    assert sorted(probe.EXPORTS) == names and len(names) == 4
+    for n in names:
+        assert hasattr(P, n), f"{n} declared in teletron_probe.h but not exported"
+        assert not hasattr(L, n)
+    for gone in ("tt_norm_stream_copy", "tt_norm_stream_probe"):
+        assert not hasattr(L, gone)
+    assert P.tt_probe_abi_version() == 1
+    assert P.tt_probe_stream_copy(None, None, 32, None) == 1
+    assert P.tt_probe_stream_copy(16, 16, 24, None) == 1                                  # not whole 16-byte pieces
+    # allocation lengths are part of the call: the third and fourth tensor read and the second written
+    # follow the first ones in the same allocations, and a call that would step outside is refused
+    KiB = 1024
+    ok = (0x10000, 8 * KiB, 0x20000, 8 * KiB, 0x30000, 8 * KiB)                          # (dst, len, a, len, b, len)
+    assert P.tt_probe_stream(*ok, 4 * KiB, 3, 1, 1, 0, 0, None) != 1 or b"need" not in P.tt_probe_last_error()
+    short = (0x10000, 4 * KiB, 0x20000, 4 * KiB, 0x30000, 4 * KiB)
+    for reads, writes in ((3, 1), (4, 2), (2, 2)):
+        assert P.tt_probe_stream(*short, 4 * KiB, reads, writes, 1, 0, 0, None) == 1
+        assert b"need allocations" in P.tt_probe_last_error()
+    assert P.tt_probe_stream(*short, 4 * KiB, 2, 1, 3, 0, 0, None) == 2                   # shape not built
+    assert P.tt_probe_stream(*short, 4 * KiB + 16, 2, 1, 1, 0, 0, None) == 1              # not whole runs
+    assert P.tt_probe_stream(*short, 4 * KiB, 0, 0, 1, 0, 0, None) == 1                   # no stream at all
+
+
+def test_wide_forms_query_matches_the_python_gate():
+    """tt_norm_wide_forms_supported: 3072 columns, or any supported row of up to 384 16-byte pieces; the
+    Python-side gate of the gated / residual Functions says the same for every width."""
+    from teletron_amd import capi
+    from teletron_amd import fusedlayers as FL
+    L = capi.lib()
+    for dt, code in ((torch.bfloat16, capi.BF16), (torch.float16, capi.F16), (torch.float32, capi.F32)):
+        for cols in list(range(0, 8200, 4)) + [3072, 3080, 1536, 1540, 8192]:
+            assert bool(L.tt_norm_wide_forms_supported(cols, code)) == FL.wide_forms_supported(cols, dt), (cols, dt)
+    assert L.tt_norm_wide_forms_supported(3072, capi.F32) == 1 and L.tt_norm_wide_forms_supported(1540, capi.F32) == 0
+    assert L.tt_norm_wide_forms_supported(3080, capi.BF16) == 0 and L.tt_norm_wide_forms_supported(3064, capi.BF16) == 1
+    assert L.tt_norm_wide_forms_supported(3072, 7) == 0
+    # beyond it the three entry points answer TT_NORM_EUNSUPPORTED before touching a pointer
+    assert L.tt_gated_residual_adaln_forward(*([None] * 9), 1, 4, 3080, 1e-6, capi.BF16, None) == 2
+    assert L.tt_gated_residual_adaln_backward(*([None] * 13), 1, 4, 4096, capi.BF16, None, 0, None) == 2
+    assert L.tt_adaln_backward_residual(*([None] * 9), 1, 4, 1540, capi.F32, None, 0, None) == 2
+    assert L.tt_gated_residual_adaln_backward_workspace_bytes(1, 4, 3080, capi.BF16) == 0
 
 
 def test_extension_modules_expose_reference_names():
