@@ -79,6 +79,9 @@ WORKLOADS = {
                                "contiguous copy, dense RMSNorm Function per tensor, then the rotary embedding as "
                                "PyTorch ops (the published apply_rotary_emb formula), torch.split's backward; same "
                                "traffic accounting as qkv-site-rope",
+    "cached-set": "the four cfg4 kernels on working sets that stay in the 256 MB last-level cache (4096 and 8192 rows x "
+                  "3072 bf16, the same buffers launch after launch): what the kernels' own instruction streams "
+                  "allow when memory is not the limit, as the per-row slope between the two sizes",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -361,6 +364,79 @@ def stream_ceiling(args, torch, capi, dev):
     }))
 
 
+def cached_set(args, torch, capi, dev):
+    """The cfg4 kernels with memory taken out of the picture as far as this part allows: 4096 and 8192 rows (25 and
+    50 MB per tensor; a backward call touches three of them), the same buffers launch after launch, so every
+    launch after the first finds its working set in the 256 MB last-level cache.  Both sizes give every one of the
+    1024 wavefronts of a backward grid whole rows (4 and 8), so the difference between them is the steady-state
+    cost of 4 rows per wavefront without the launch, the parameter loads and the final reduction; scaled to the
+    116 rows per wavefront of the full problem it says how fast the kernel's own instruction stream could go."""
+    L = capi.lib()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    bf = torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    big = 8192
+    x = torch.randn(big, COLS, device=dev, generator=gen).to(bf)
+    g = torch.randn(big, COLS, device=dev, generator=gen).to(bf)
+    w = (1 + 0.02 * torch.randn(COLS, device=dev, generator=gen)).to(bf)
+    sc, sh = ((0.1 * torch.randn(1, COLS, device=dev, generator=gen)).to(bf) for _ in range(2))
+    out, dx = torch.empty_like(x), torch.empty_like(x)
+    rstd, mean = (torch.empty(big, device=dev, dtype=torch.float32) for _ in range(2))
+    dw, dsc, dsh = torch.empty_like(w), torch.empty_like(sc), torch.empty_like(sc)
+    n = max(L.tt_rmsnorm_backward_workspace_bytes(big, COLS, capi.BF16),
+            L.tt_adaln_backward_workspace_bytes(1, big, COLS, capi.BF16))
+    ws = torch.empty(n, device=dev, dtype=torch.uint8)
+
+    def calls(rows):
+        return {
+            "rmsnorm_forward": (2, lambda: L.tt_rmsnorm_forward(p(out), p(rstd), p(x), p(w), rows, COLS, EPS, capi.BF16, stream)),
+            "rmsnorm_backward": (3, lambda: L.tt_rmsnorm_backward(p(dx), p(dw), p(g), p(x), p(w), p(rstd), rows, COLS,
+                                                                  capi.BF16, p(ws), n, stream)),
+            "adaln_forward": (2, lambda: L.tt_adaln_forward(p(out), p(mean), p(rstd), p(x), p(sc), p(sh), 1, rows, COLS, EPS,
+                                                            capi.BF16, stream)),
+            "adaln_backward": (3, lambda: L.tt_adaln_backward(p(dx), p(dsc), p(dsh), p(g), p(x), p(sc), p(mean), p(rstd), 1,
+                                                              rows, COLS, capi.BF16, p(ws), n, stream)),
+        }
+
+    def timed(fn):
+        for _ in range(max(5, args.warmup)):
+            if fn() != 0:
+                raise RuntimeError(L.tt_norm_last_error().decode())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps * 1e3
+
+    # forward calls first so that rstd / mean hold real statistics for the backward ones
+    small, large = calls(big // 2), calls(big)
+    res = {}
+    for name in ("rmsnorm_forward", "adaln_forward", "rmsnorm_backward", "adaln_backward"):
+        mult = large[name][0]
+        t_large = timed(large[name][1])
+        t_small = timed(small[name][1])
+        slope = (t_large - t_small) / (big // 2)                    # us per row, all wavefronts working
+        full = slope * ROWS
+        res[name] = {"us_4096_rows": round(t_small, 2), "us_8192_rows": round(t_large, 2),
+                     "us_per_1024_rows": round(slope * 1024, 3),
+                     "cfg4_us_at_this_rate": round(full, 1),
+                     "GB/s_at_this_rate": round(mult * ROWS * COLS * 2 / full / 1e3, 0),
+                     "frac_of_hbm_peak_at_this_rate": round(mult * ROWS * COLS * 2 / full / 1e3 / HBM_PEAK_GBS, 3)}
+    worst = min(res.values(), key=lambda r: r["GB/s_at_this_rate"])
+    print(json.dumps({
+        "metric": "rate of the cfg4 kernels on a cache-resident working set (instruction-stream ceiling), GB/s equivalent",
+        "value": worst["GB/s_at_this_rate"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sum(r["us_8192_rows"] for r in res.values()) / 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": WORKLOADS["cached-set"], "rows": [big // 2, big], "cols": COLS},
+        "kernels": res,
+    }))
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -383,7 +459,18 @@ def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
     import torch
     from oracle import norm_oracle as O
 
+    # every core the box gives this process (its CPU share), as intra-op threads
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    limit = os.environ.get("OMP_NUM_THREADS")
+    threads = min(cores, int(limit)) if limit and limit.isdigit() else cores
+    torch.set_num_threads(threads)
     threads = torch.get_num_threads()
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            cpu_model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "unknown")
+    except OSError:
+        pass
     r = O.make_rmsnorm_inputs((1, sample_rows), COLS, torch.bfloat16, seed=0)
     a = O.make_adaln_inputs(1, sample_rows, COLS, torch.bfloat16, seed=0)
 
@@ -410,7 +497,8 @@ def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
         if k >= 3:
             t1.append(time.perf_counter() - t0)
     m1 = sorted(t1)[len(t1) // 2]
-    cfg1 = {"value": round(5 * 8192 * COLS * 4 / m1 / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+    cfg1 = {"value": round(5 * 8192 * COLS * 4 / m1 / 1e9, 3), "unit": "GB/s", "cores": threads, "threads": threads,
+            "cpu_model": cpu_model, "kind": "port",
             "ms_per_pass": round(m1 * 1e3, 2),
             "sample": "config 1 in full: RMSNorm fwd+bwd, x [2, 4096, 3072] fp32, PyTorch CPU eager (oracle "
                       "restatement), 3 warm-up + 10 timed passes, median"}
@@ -418,6 +506,9 @@ def cpu_eager_baseline(sample_rows: int = ROWS, reps: int = 5):
         "value": round(nbytes / t / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "threads": threads,
+        "cpu_model": cpu_model,
+        "host_cpus": os.cpu_count(),
         "kind": "port",
         "sample": f"{sample_rows} of {ROWS} rows x {COLS} bf16, RMSNorm + AdaLN fwd+bwd via PyTorch CPU eager "
                   f"(oracle restatement), median of {reps}, {t * 1e3:.1f} ms per pass",
@@ -441,6 +532,9 @@ def main():
     L = capi.lib()
     if args.workload == "stream-ceiling":
         stream_ceiling(args, torch, capi, dev)
+        return
+    if args.workload == "cached-set":
+        cached_set(args, torch, capi, dev)
         return
     calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)
     headline = args.workload == "cfg4"

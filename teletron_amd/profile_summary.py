@@ -10,7 +10,9 @@ kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for 
     python -m teletron_amd.profile_summary stream --dir rocprof_out        (<dir>/stream.json, <dir>/stream_stall)
     python -m teletron_amd.profile_summary variants --dir rocprof_out      (<dir>/variant_<name>.json, _sq, _stall)
     python -m teletron_amd.profile_summary runs --dir rocprof_out          (<dir>/run_<name>_<workload>.json, run_<name>_trace)
+    python -m teletron_amd.profile_summary cached --dir rocprof_out        (<dir>/cached_<name>.json)
 
+`python -m teletron_amd.profile_collect <what> --dir <dir>` runs the commands that produce those inputs.
 The databases are large; run this where they were written and keep only what it writes (--out).
 """
 from __future__ import annotations
@@ -197,7 +199,7 @@ fp32 partial column sums (256 workgroups x 12 or 24 KiB).
         f.write(md)
     print("wrote profiles/bench_cfg4_all_kernels.md, profiles/cfg4_traffic.json (digest %s)" % digest)
 
-    passes = {p: os.path.join(directory, p) for p in ("sq", "tcc", "stall") if os.path.isdir(os.path.join(directory, p))}
+    passes = {p: os.path.join(directory, p) for p in CFG4_PASSES if os.path.isdir(os.path.join(directory, p))}
     if passes:
         cfg4_counters(passes, digest)
 
@@ -208,7 +210,11 @@ PASS_COUNTERS = {
     "tcc": "TCC_HIT_sum TCC_MISS_sum TCC_EA0_RDREQ_sum TCC_EA0_WRREQ_sum",
     "stall": "TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum TCC_EA0_WRREQ_STALL_sum "
              "TCC_TOO_MANY_EA_WRREQS_STALL_sum",
+    # the two passes taken per tuning variant
+    "variant_sq": "SQ_WAVES SQ_INSTS_VALU SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY",
+    "variant_stall": "TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum",
 }
+CFG4_PASSES = ("sq", "tcc", "stall")
 
 
 def cfg4_counters(passes, digest):
@@ -341,10 +347,45 @@ persistent form (256 / 1024 workgroups), anything larger the one-shot form.  Ave
 
 {chr(10).join(lines)}
 """
+    traffic_md = ""
+    fd, wd = os.path.join(directory, "stream_fetch"), os.path.join(directory, "stream_write")
+    if os.path.isdir(fd) and os.path.isdir(wd):
+        cf, cw = counters(fd, by_grid=True), counters(wd, by_grid=True)
+        kib = CFG4_TENSOR / 1024
+        f_scale = kib / next(v["FETCH_SIZE"] for (k, _), v in cf.items() if k.startswith("stream_copy_kernel"))
+        w_scale = kib / next(v["WRITE_SIZE"] for (k, _), v in cw.items() if k.startswith("stream_copy_kernel"))
+        lines = ["| kernel | grid (threads) | tensors read | read MB (FETCH_SIZE, scaled) | per tensor claimed | tensors "
+                 "written | written MB (WRITE_SIZE, scaled) | per tensor claimed |", "|---|---|---|---|---|---|---|---|"]
+        worst = 0.0
+        for (k, grid), v in sorted(cf.items()):
+            m = re.match(r"stream_probe_kernel<(\d+), (\d+), (\d+), (\d+)>", k)
+            if not m or (k, grid) not in cw:
+                continue
+            nr, nw = int(m.group(1)), int(m.group(2))
+            rb = v["FETCH_SIZE"] * f_scale * 1024
+            wb = cw[(k, grid)]["WRITE_SIZE"] * w_scale * 1024
+            pr = rb / nr / CFG4_TENSOR if nr else float("nan")
+            pw = wb / nw / CFG4_TENSOR if nw else float("nan")
+            worst = max(worst, abs(pr - 1) if nr else 0.0, abs(pw - 1) if nw else 0.0)
+            lines.append(f"| `{k}` | {grid} | {nr} | {rb / 1e6:.1f} | {pr:.3f} | {nw} | {wb / 1e6:.1f} | {pw:.3f} |")
+        traffic_md = f"""
+## The probes move the bytes they claim (FETCH_SIZE / WRITE_SIZE passes over the same probes)
+
+    rocprofv3 --pmc FETCH_SIZE -d {DIR_SHOWN}/stream_fetch -o r -- python3 bench.py --workload stream-ceiling --steps 3 --warmup 4
+    rocprofv3 --pmc WRITE_SIZE -d {DIR_SHOWN}/stream_write -o r -- python3 bench.py --workload stream-ceiling --steps 3 --warmup 4
+
+Counters scaled by what they read for `stream_copy_kernel` in the same run (729.9 MB read and written:
+FETCH_SIZE x {f_scale:.3f}, WRITE_SIZE x {w_scale:.3f} KiB).  "Per tensor claimed" = measured bytes / (tensors x 729.9 MB):
+1.000 means the probe's HBM traffic is exactly the streams its bandwidth figure is computed from (largest
+deviation in this table: {100 * worst:.1f} %).  What each launch writes is also checked value by value
+(`tests/test_gpu_probe.py`).
+
+{chr(10).join(lines)}
+"""
     md = f"""# Streaming ceiling: what this memory system gives each read/write mix
 
 {BOX}.  Kernel sources digest `{digest}`.  `python3 bench.py --workload stream-ceiling --steps {b['steps']} --warmup {b['warmup']}`:
-plain streams over 729.9 MB tensors through the library's probe kernel (`tt_norm_stream_probe`: non-temporal
+plain streams over 729.9 MB tensors through the probe library's kernel (`tt_probe_stream` of libteletron_probe.so: non-temporal
 16-byte loads, one contiguous run per wavefront and tensor, no arithmetic beyond one add), {b['steps']} launches back
 to back between two events.  Written by `python -m teletron_amd.profile_summary stream --dir {DIR_SHOWN}`.
 
@@ -362,7 +403,7 @@ run faster than it (see bench_cfg4_all_kernels.md).
 {chr(10).join(rows)}
 
 {chr(10).join(others)}
-{stall_md}"""
+{stall_md}{traffic_md}"""
     with open(os.path.join(PROFILES, "stream_ceiling.md"), "w") as f:
         f.write(md)
     print("wrote profiles/stream_ceiling.md")
@@ -370,20 +411,31 @@ run faster than it (see bench_cfg4_all_kernels.md).
 
 # --------------------------------------------------------------------------------------- variants
 
-VARIANTS = [  # name, build flags, what it changes
-    ("base", "", "the shipped kernels"),
-    ("nodrain", "--flag=-DTTN_BWD_DRAIN_STORES=0",
+VARIANTS = [  # name, hipcc flags of the build ([] = the shipped library), what it changes
+    ("base", [], "the shipped kernels"),
+    ("unpacked", ["-DTTN_BWD_PACKED_MATH=0"],
+     "backward: every product and column sum on unpacked fp32 values (unpack, multiply, convert, unpack again), as "
+     "before the packed dot-product forms"),
+    ("packedproducts", ["-DTTN_BWD_PACKED_MATH=1"],
+     "backward: gy / gx = rnd(g * parameter) from packed pairs; the column sums still unpack g"),
+    ("nodrain", ["-DTTN_BWD_DRAIN_STORES=0"],
      "backward: a row's first pass waits for its own loads only, not for the previous row's stores"),
-    ("plainstore", "--flag=-DTTN_RMS_BWD_STORE=0 --flag=-DTTN_ADALN_BWD_STORE=0",
+    ("plainstore", ["-DTTN_RMS_BWD_STORE=0", "-DTTN_ADALN_BWD_STORE=0"],
      "backward: plain streaming stores instead of write-through"),
-    ("fullahead", "--flag=-DTTN_RMS_BWD_PREFETCH_MID=0 --flag=-DTTN_ADALN_BWD_PREFETCH_MID=0",
+    ("fullahead", ["-DTTN_RMS_BWD_PREFETCH_MID=0", "-DTTN_ADALN_BWD_PREFETCH_MID=0"],
      "backward: the next row is requested before the current one is processed (a full row ahead)"),
-    ("onebuffer", "--flag=-DTTN_RMS_BWD_ROW_BUFFERS=1 --flag=-DTTN_ADALN_BWD_ROW_BUFFERS=1",
+    ("onebuffer", ["-DTTN_RMS_BWD_ROW_BUFFERS=1", "-DTTN_ADALN_BWD_ROW_BUFFERS=1"],
      "backward: one row buffer, no prefetch"),
-    ("twowaves", "--flag=-DTTN_BWD_WAVES_PER_SIMD=2 '--flag=-DTTN_RMS_BWD_BLOCKS_PER_CU=(C>=1024?2:3)' "
-                 "'--flag=-DTTN_ADALN_BWD_BLOCKS_PER_CU=(C>=1024?2:3)'",
+    ("twowaves", ["-DTTN_BWD_WAVES_PER_SIMD=2", "-DTTN_RMS_BWD_BLOCKS_PER_CU=(C>=1024?2:3)",
+                  "-DTTN_ADALN_BWD_BLOCKS_PER_CU=(C>=1024?2:3)"],
      "backward: two workgroups per compute unit (two wavefronts per SIMD, half the registers each)"),
-    ("fwd5", "'--flag=-DTTN_RMS_FWD_DYN_LDS=(C>=1024?(sizeof(T)==2?0:76800):0)'",
+    ("loadcached", ["-DTTN_BWD_LOAD_POLICY=0"],
+     "backward: row loads without the non-temporal hint (buffer loads, default cache policy)"),
+    ("loadsystem", ["-DTTN_BWD_LOAD_POLICY=19"],
+     "backward: row loads marked sc0 sc1 nt (system scope + non-temporal)"),
+    ("grid88", ["-DTTN_BWD_GRID_PERCENT=88"],
+     "backward: persistent grid over 88 % of the compute units (226 workgroups instead of 256)"),
+    ("fwd5", ["-DTTN_RMS_FWD_DYN_LDS=(C>=1024?(sizeof(T)==2?0:76800):0)"],
      "RMSNorm forward: no occupancy throttle (five one-shot workgroups per compute unit instead of three)"),
 ]
 
@@ -393,9 +445,11 @@ def variants(directory):
     calls = ["rmsnorm_forward", "rmsnorm_backward", "adaln_forward", "adaln_backward"]
     rows = ["| variant | ms per step | GB/s | % of 8 TB/s | " + " | ".join(c + " µs" for c in calls) + " |",
             "|---|---|---|---|" + "---|" * len(calls)]
-    ctr = ["| variant | kernel | SQ_WAIT_INST_ANY | SQ_ACTIVE_INST_ANY | SQ_BUSY_CYCLES | WRREQ_DRAM_CREDIT_STALL | "
-           "RDREQ_DRAM_CREDIT_STALL |", "|---|---|---|---|---|---|---|"]
+    ctr = ["| variant | kernel | VALU instructions per row | SQ_ACTIVE_INST_ANY / SQ_WAVE_CYCLES | SQ_WAIT_INST_ANY / "
+           "SQ_WAVE_CYCLES | SQ_INSTS_VALU | SQ_ACTIVE_INST_ANY | SQ_WAIT_INST_ANY | SQ_WAVE_CYCLES | SQ_BUSY_CYCLES | "
+           "WRREQ_DRAM_CREDIT_STALL | RDREQ_DRAM_CREDIT_STALL |", "|---|---|---|---|---|---|---|---|---|---|---|---|"]
     cmds = []
+    vdir = f"{DIR_SHOWN}/variants"
     for name, flags, what in VARIANTS:
         bj = os.path.join(directory, f"variant_{name}.json")
         if not os.path.exists(bj):
@@ -403,28 +457,35 @@ def variants(directory):
         b = json.loads(open(bj).read().strip().splitlines()[-1])
         rows.append(f"| `{name}` | {b['ms_per_step']:.4f} | {b['value']:.0f} | {100 * b['frac_of_hbm_peak']:.1f} | "
                     + " | ".join(f"{b['per_call_untimed'][c]['median_us']:.1f}" for c in calls) + " |")
-        cmds.append(f"* `{name}`: {what}" + (f"  \n  `python -m teletron_amd.build --variant /tmp/lib_{name}.so {flags}`" if flags else ""))
+        build = " ".join(f"'--flag={f}'" for f in flags)
+        cmds.append(f"* `{name}`: {what}" + (f"  \n  `python -m teletron_amd.build --variant {vdir}/lib_{name}.so {build}`" if flags else ""))
         merged = {}
         for p in ("sq", "stall"):
             d = os.path.join(directory, f"variant_{name}_{p}")
             if os.path.isdir(d):
                 for k, v in counters(d).items():
                     merged.setdefault(k, {}).update(v)
+        nan = float("nan")
         for k, v in sorted(merged.items()):
             if "bwd_kernel<bf16_t, 3072" in k and "SQ_WAIT_INST_ANY" in v:
-                ctr.append(f"| `{name}` | `{k.split('<')[0]}` | {v['SQ_WAIT_INST_ANY']:,.0f} | {v['SQ_ACTIVE_INST_ANY']:,.0f} | "
-                           f"{v['SQ_BUSY_CYCLES']:,.0f} | {v.get('TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum', float('nan')):,.0f} | "
-                           f"{v.get('TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum', float('nan')):,.0f} |")
+                wc = v.get("SQ_WAVE_CYCLES", nan)
+                ctr.append(f"| `{name}` | `{k.split('<')[0]}` | {v.get('SQ_INSTS_VALU', nan) / CFG4_ROWS:.0f} | "
+                           f"{v['SQ_ACTIVE_INST_ANY'] / wc:.2f} | {v['SQ_WAIT_INST_ANY'] / wc:.2f} | "
+                           f"{v.get('SQ_INSTS_VALU', nan):,.0f} | {v['SQ_ACTIVE_INST_ANY']:,.0f} | {v['SQ_WAIT_INST_ANY']:,.0f} | "
+                           f"{wc:,.0f} | {v['SQ_BUSY_CYCLES']:,.0f} | "
+                           f"{v.get('TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum', nan):,.0f} | "
+                           f"{v.get('TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum', nan):,.0f} |")
     md = f"""# Tuning variants of the cfg4 step: what each pipeline choice is worth (bench.py, 118 800 x 3072 bf16)
 
 {BOX}.  Kernel sources digest `{digest}`.  Each variant is the shipped kernel source built with other values of
-the tuning macros at the top of `rmsnorm.hip` / `adaln.hip`, loaded in place of the shipped library, and run
-through the unchanged benchmark on one box, one after the other:
+the tuning macros at the top of `rmsnorm.hip` / `adaln.hip`, loaded in place of the shipped library
+(`TELETRON_AMD_LIB` in the environment of the command), and run through the unchanged benchmark on one box, one
+after the other, by `python -m teletron_amd.profile_collect variants --dir {DIR_SHOWN}`:
 
-    python -m teletron_amd.build --variant /tmp/lib_<name>.so <flags>
-    TELETRON_AMD_LIB=/tmp/lib_<name>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline
-    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY -d {DIR_SHOWN}/variant_<name>_sq -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
-    TELETRON_AMD_LIB=/tmp/lib_<name>.so rocprofv3 --pmc TCC_EA0_WRREQ_DRAM_CREDIT_STALL_sum TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum -d {DIR_SHOWN}/variant_<name>_stall -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+    python -m teletron_amd.build --variant {vdir}/lib_<name>.so <flags>
+    TELETRON_AMD_LIB={vdir}/lib_<name>.so  python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline
+    TELETRON_AMD_LIB={vdir}/lib_<name>.so  rocprofv3 --pmc {PASS_COUNTERS['variant_sq']} -d {DIR_SHOWN}/variant_<name>_sq -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
+    TELETRON_AMD_LIB={vdir}/lib_<name>.so  rocprofv3 --pmc {PASS_COUNTERS['variant_stall']} -d {DIR_SHOWN}/variant_<name>_stall -o r -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline
 
 {chr(10).join(cmds)}
 
@@ -433,23 +494,72 @@ Per-call figures are HIP-event medians over 30 untimed steps.  Written by
 
 {chr(10).join(rows)}
 
-Counters of the two backward row kernels, per dispatch (averages):
+Counters of the two backward row kernels, per dispatch (averages; the SQ cycle counters tick once per four
+clocks; VALU instructions per row = SQ_INSTS_VALU / 118 800):
 
 {chr(10).join(ctr)}
 
-Reading: every alternative keeps more requests in flight per wavefront than the shipped pipeline (or, for
-`onebuffer`, fewer) and is slower; the slower ones show more DRAM-credit stall cycles at the L2-to-memory
-interface, i.e. the extra requests queue instead of being served.  None reaches the 80 % line; see
-stream_ceiling.md for what plain streams of the same read/write mix reach.
+Reading.  Arithmetic: `unpacked` -> `packedproducts` -> `base` removes about a quarter of the backward kernels'
+vector instructions (and with them that share of the cycles in which the one wavefront of a SIMD is issuing),
+and the kernels' duration does not follow: the time goes to waiting instead (SQ_WAIT_INST_ANY grows by what
+SQ_ACTIVE_INST_ANY loses).  The backward kernels are not limited by instruction issue.  Memory pipeline: every
+alternative keeps more requests in flight per wavefront than the shipped pipeline (or, for `onebuffer`, fewer) and
+is slower; the slower ones show more DRAM-credit stall cycles at the L2-to-memory interface, i.e. the extra
+requests queue instead of being served.  Loads without the non-temporal hint cost 10 %; no other cache policy
+of the loads, and no smaller grid, gains anything.  None reaches the 80 % line; see stream_ceiling.md for what
+plain streams of the same read/write mix reach.
 """
     with open(os.path.join(PROFILES, "bench_cfg4_tuning_variants.md"), "w") as f:
         f.write(md)
     print("wrote bench_cfg4_tuning_variants.md")
 
 
+def cached(directory):
+    """bench.py --workload cached-set for the shipped library and the build without the packed forms."""
+    digest = kernel_source_digest()
+    names = {"base": "shipped (packed dot-product forms)", "unpacked": "`-DTTN_BWD_PACKED_MATH=0` (unpacked fp32 arithmetic)"}
+    rows = ["| build | kernel | µs at 4096 rows | µs at 8192 rows | µs per 1024 rows (slope) | 118 800 rows at that rate, µs | "
+            "GB/s equivalent | % of 8 TB/s |", "|---|---|---|---|---|---|---|---|"]
+    steps = None
+    for name, label in names.items():
+        f = os.path.join(directory, f"cached_{name}.json")
+        if not os.path.exists(f):
+            continue
+        b = json.loads(open(f).read().strip().splitlines()[-1])
+        steps = (b["steps"], b["warmup"])
+        for k, r in b["kernels"].items():
+            rows.append(f"| {label} | `{k}` | {r['us_4096_rows']:.2f} | {r['us_8192_rows']:.2f} | {r['us_per_1024_rows']:.3f} | "
+                        f"{r['cfg4_us_at_this_rate']:.1f} | {r['GB/s_at_this_rate']:.0f} | "
+                        f"{100 * r['frac_of_hbm_peak_at_this_rate']:.0f} |")
+    vdir = f"{DIR_SHOWN}/variants"
+    md = f"""# The cfg4 kernels on a cache-resident working set: what their instruction streams allow
+
+{BOX}.  Kernel sources digest `{digest}`.  `bench.py --workload cached-set` launches each of the four cfg4 calls back
+to back on the same buffers at 4096 and at 8192 rows x 3072 bf16 (25 / 50 MB per tensor, at most three tensors
+per call): after the first launch the working set sits in the 256 MB last-level cache, so the memory
+system answers faster than HBM can.  Both sizes give each of the 1024 wavefronts of a backward grid whole rows
+(4 and 8); the difference between the two is the steady-state cost of 4 more rows per wavefront, free of launch,
+parameter loads and the final reduction.  Scaled to the full problem it is the duration the kernel would have if
+HBM delivered like the cache -- an upper bound on what fewer instructions could buy.  Collected by
+`python -m teletron_amd.profile_collect cached --dir {DIR_SHOWN}`:
+
+    python3 bench.py --workload cached-set --steps {steps[0] if steps else 200} --warmup {steps[1] if steps else 20}
+    python -m teletron_amd.build --variant {vdir}/lib_unpacked.so '--flag=-DTTN_BWD_PACKED_MATH=0'
+    TELETRON_AMD_LIB={vdir}/lib_unpacked.so  python3 bench.py --workload cached-set --steps {steps[0] if steps else 200} --warmup {steps[1] if steps else 20}
+
+Written by `python -m teletron_amd.profile_summary cached --dir {DIR_SHOWN}`.
+
+{chr(10).join(rows)}
+"""
+    with open(os.path.join(PROFILES, "cached_set_instruction_ceiling.md"), "w") as f:
+        f.write(md)
+    print("wrote cached_set_instruction_ceiling.md")
+
+
 # ------------------------------------------------------------------- run length at the QK-norm site
 
-RUN_VARIANTS = [("run1", 1), ("run3", 3), ("base", 6), ("run12", 12)]
+RUN_LENGTHS = (1, 3, 6, 12)   # 6 is what ships; built explicitly like the others so that all four are measured alike
+RUN_VARIANTS = [(f"run{n}", n) for n in RUN_LENGTHS]
 RUN_WORKLOADS = ["cfg2-strided-rope", "cfg2-strided"]
 
 
@@ -477,7 +587,7 @@ def run_lengths(directory):
                     elif "bwd_kernel" in r["name"]:
                         bwd = r["avg_us"]
         c = js["cfg2-strided"]["per_call_untimed"]
-        rows.append(f"| {run}{' (shipped)' if name == 'base' else ''} | {js['cfg2-strided-rope']['ms_per_step']:.4f} | {fwd:.1f} | "
+        rows.append(f"| {run}{' (shipped)' if run == 6 else ''} | {js['cfg2-strided-rope']['ms_per_step']:.4f} | {fwd:.1f} | "
                     f"{bwd:.1f} | {js['cfg2-strided']['ms_per_step']:.4f} | "
                     f"{c['rmsnorm_forward_strided_q']['median_us']:.1f} / {c['rmsnorm_backward_strided_q']['median_us']:.1f} |")
     md = f"""# Run length of the strided QK-norm kernels: heads a wavefront takes per table fetch
@@ -488,12 +598,12 @@ rotary kernels fetch the token's cos/sin rows once per run, the backward kernels
 per run; the forward kernel without tables always takes single groups.  With 1 every row fetches its own 1 KiB of
 tables (what the kernels did before runs existed).  29 700 tokens x 24 heads x 128, bf16, q and k through the C ABI
 (`cfg2-strided-rope`: the strided norm with the rotation, forward and backward; `cfg2-strided`: without), one box, one
-after the other:
+after the other, by `python -m teletron_amd.profile_collect runs --dir {DIR_SHOWN}`:
 
-    python -m teletron_amd.build --variant /tmp/lib_run<N>.so --flag=-DTTN_STRIDED_RUN=<N>
-    TELETRON_AMD_LIB=/tmp/lib_run<N>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided-rope
-    TELETRON_AMD_LIB=/tmp/lib_run<N>.so python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided
-    TELETRON_AMD_LIB=/tmp/lib_run<N>.so rocprofv3 --kernel-trace --stats -d {DIR_SHOWN}/run_<name>_trace -o bench -- python3 bench.py --steps 30 --warmup 5 --no-cpu-baseline --workload cfg2-strided-rope
+    python -m teletron_amd.build --variant {DIR_SHOWN}/variants/lib_run<N>.so --flag=-DTTN_STRIDED_RUN=<N>
+    TELETRON_AMD_LIB={DIR_SHOWN}/variants/lib_run<N>.so  python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided-rope
+    TELETRON_AMD_LIB={DIR_SHOWN}/variants/lib_run<N>.so  python3 bench.py --steps 50 --warmup 10 --no-cpu-baseline --workload cfg2-strided
+    TELETRON_AMD_LIB={DIR_SHOWN}/variants/lib_run<N>.so  rocprofv3 --kernel-trace --stats -d {DIR_SHOWN}/run_run<N>_trace -o bench -- python3 bench.py --steps 30 --warmup 5 --no-cpu-baseline --workload cfg2-strided-rope
 
 Kernel columns are rocprofv3 averages of `rmsnorm_fwd_kernel<bf16_t, 128, Strided3Rows, RopeTable>` and the matching
 backward kernel.  Written by `python -m teletron_amd.profile_summary runs --dir {DIR_SHOWN}`.
@@ -508,14 +618,15 @@ backward kernel.  Written by `python -m teletron_amd.profile_summary runs --dir 
 def main():
     global PROFILES, DIR_SHOWN
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs"))
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs", "cached"))
     ap.add_argument("--dir", default="rocprof_out", help="where rocprofv3 wrote (its -d arguments' parent)")
     ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
     a = ap.parse_args()
     PROFILES = a.out
     DIR_SHOWN = a.dir.rstrip("/")
     os.makedirs(PROFILES, exist_ok=True)
-    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": run_lengths}[a.what](a.dir)
+    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": run_lengths,
+     "cached": cached}[a.what](a.dir)
 
 
 if __name__ == "__main__":
