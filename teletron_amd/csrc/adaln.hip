@@ -82,6 +82,11 @@
 #ifndef TTN_BWD_LOAD_POLICY
 #define TTN_BWD_LOAD_POLICY -1
 #endif
+// Measurement only (results are wrong): rows are read and written modulo this count, so that the working set of
+// a full-size launch stays in the L2 (1024) or the last-level cache; 0 = off.
+#ifndef TTN_BWD_ROW_WRAP
+#define TTN_BWD_ROW_WRAP 0
+#endif
 // Share of the compute units the persistent backward grids at 3072 columns cover, in per cent.
 #ifndef TTN_BWD_GRID_PERCENT
 #define TTN_BWD_GRID_PERCENT 100
@@ -346,8 +351,13 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     auto fetch = [&](RowRegs &b, int64_t grp) {
         const int64_t rs = grp * RPW + sub;  // row inside the sample
         b.ok = rs < rows_per_sample;
+#if TTN_BWD_ROW_WRAP > 0
+        b.row = lay.row(smp, rs % TTN_BWD_ROW_WRAP);
+        b.first = lay.row(smp, (grp * RPW) % TTN_BWD_ROW_WRAP) * C;
+#else
         b.row = lay.row(smp, rs);
         b.first = lay.row(smp, grp * RPW) * C;
+#endif
         const u32x4 *pg = reinterpret_cast<const u32x4 *>(g + b.row * C) + l;
         const u32x4 *px = reinterpret_cast<const u32x4 *>(xin + b.row * C) + l;
 #if TTN_BWD_LOAD_POLICY >= 0

@@ -53,6 +53,11 @@
 #ifndef TTN_BWD_LOAD_POLICY
 #define TTN_BWD_LOAD_POLICY -1
 #endif
+// Measurement only (results are wrong): rows are read and written modulo this count, so that the working set of
+// a full-size launch stays in the L2 (1024) or the last-level cache; 0 = off.
+#ifndef TTN_BWD_ROW_WRAP
+#define TTN_BWD_ROW_WRAP 0
+#endif
 // Share of the compute units the persistent backward grids at 3072 columns cover, in per cent.
 #ifndef TTN_BWD_GRID_PERCENT
 #define TTN_BWD_GRID_PERCENT 100
@@ -332,8 +337,13 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     auto fetch = [&](RowRegs &b, int64_t at_step) {
         RowAddr at, at0;
         if constexpr (kRun == 1) {
+#if TTN_BWD_ROW_WRAP > 0
+            at = map.template locate<RPW>(at_step % (TTN_BWD_ROW_WRAP / RPW), sub, C);
+            at0 = map.template locate<RPW>(at_step % (TTN_BWD_ROW_WRAP / RPW), 0, C);
+#else
             at = map.template locate<RPW>(at_step, sub, C);
             at0 = map.template locate<RPW>(at_step, 0, C);
+#endif
         } else {
             const int h = (int)(at_step % kRun);
             const int64_t first = ((at_step / kRun) * waves + me) * kRun;

@@ -24,7 +24,7 @@ import sys
 import time
 
 from teletron_amd.build import ROOT
-from teletron_amd.profile_summary import PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WORKLOAD_INFO
+from teletron_amd.profile_summary import CACHED_VARIANTS, PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WORKLOAD_INFO
 
 BENCH = ["python3", "bench.py"]
 QUICK = ["--steps", "3", "--warmup", "1", "--no-cpu-baseline"]
@@ -128,12 +128,13 @@ def runs(directory, only):
 
 
 def cached(directory, only):
-    table = [v for v in VARIANTS if v[0] in ("base", "unpacked")]
-    vdir = _build_variants(directory, table, only)
-    for name, flags, _ in table:
-        env = {"TELETRON_AMD_LIB": os.path.join(vdir, f"lib_{name}.so")} if flags else None
-        run([*BENCH, "--workload", "cached-set", "--steps", "200", "--warmup", "20"],
-            out=os.path.join(directory, f"cached_{name}.json"), env=env)
+    # (a) small working sets through the shipped library; (b) the full-size step with the backward kernels'
+    # rows wrapped to 1024 (timing only: every wavefront re-reads and re-writes one row, which stays in L2)
+    run([*BENCH, "--workload", "cached-set", "--steps", "200", "--warmup", "20"], out=os.path.join(directory, "cached_rows.json"))
+    vdir = _build_variants(directory, CACHED_VARIANTS, only)
+    for name, _, _ in CACHED_VARIANTS:
+        run([*BENCH, "--steps", "50", "--warmup", "10", "--no-cpu-baseline"], out=os.path.join(directory, f"cached_{name}.json"),
+            env={"TELETRON_AMD_LIB": os.path.join(vdir, f"lib_{name}.so")})
 
 
 def main():
