@@ -672,7 +672,7 @@ static int wide_form_unsupported(const char *who, int64_t cols) {
 // The rows a wavefront handles together (up to eight when rows are narrow) are addressed with 32-bit
 // byte offsets from the first of them; in the sequence-first layout they lie batch rows apart.
 static int check_seq_first(const char *who, int64_t batch, int64_t cols, int dtype) {
-    if (batch * cols * (int64_t)elem_bytes(dtype) > (int64_t)(1 << 28))
+    if (batch * cols * (int64_t)elem_bytes(dtype) > kMaxRowStrideBytes)
         return fail(TT_NORM_EINVAL, "%s: batch * cols * element size exceeds 256 MiB", who);
     return TT_NORM_OK;
 }

@@ -35,6 +35,7 @@ struct PadGeom {
     static constexpr int LANES = LANES_;
     static constexpr int CHUNKS = CHUNKS_;
     static constexpr int RPW = kWaveSize / LANES;
+    static_assert(LANES >= kMinRowLanes, "the host's row-stride cap assumes at most kMaxRowsPerWave rows per wavefront");
     static_assert(LANES == 8 || LANES == 16 || LANES == 32 || LANES == 64, "row must fill an aligned lane group");
     static_assert(LANES == 64 || CHUNKS == 1, "only full wavefronts take several accesses per lane");
 };

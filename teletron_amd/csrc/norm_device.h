@@ -37,6 +37,14 @@ struct f16_t {
 
 constexpr int kWaveSize = 64;
 constexpr int kRowWaves = 4;  // wavefronts per workgroup of every row kernel
+// The narrowest row geometry any kernel is instantiated with (tuned: 16 lanes; any-width: 8), hence the most rows
+// one wavefront handles together.  Rows of a wavefront are addressed with 32-bit byte offsets from the first of
+// them, so (kMaxRowsPerWave - 1) row strides must stay below 4 GiB: the host caps a row stride at kMaxRowStrideBytes.
+constexpr int kMinRowLanes = 8;
+constexpr int kMaxRowsPerWave = kWaveSize / kMinRowLanes;
+constexpr int64_t kMaxRowStrideBytes = (int64_t)1 << 28;
+static_assert((kMaxRowsPerWave - 1) * kMaxRowStrideBytes + (1 << 20) < ((int64_t)1 << 32),
+              "rows of one wavefront must stay within a 32-bit byte offset of the first");
 constexpr int kRowThreads = kRowWaves * kWaveSize;
 
 // Caps a kernel's register use so that at least N wavefronts fit on each SIMD

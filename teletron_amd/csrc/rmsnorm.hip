@@ -681,9 +681,10 @@ static int check_strided(const char *who, int64_t n0, int64_t n1, int64_t n2, in
         if (s < 0 || s % vec != 0)
             return fail(TT_NORM_EALIGN, "%s: %s stride %lld is not a non-negative multiple of %lld elements (16 bytes)",
                         who, what, (long long)s, (long long)vec);
-    // the rows one wavefront handles together (up to four consecutive indices of the last dimension)
-    // are addressed with 32-bit byte offsets from the first of them
-    if (strides[2] > (int64_t)(1 << 28) / (int64_t)elem_bytes(dtype))
+    // the rows one wavefront handles together (up to kMaxRowsPerWave consecutive indices of the last dimension:
+    // eight for the narrowest any-width rows, four for 128 two-byte columns, two for 128 four-byte ones) are
+    // addressed with 32-bit byte offsets from the first of them: (kMaxRowsPerWave - 1) * stride < 4 GiB
+    if (strides[2] > kMaxRowStrideBytes / (int64_t)elem_bytes(dtype))
         return fail(TT_NORM_EINVAL, "%s: %s stride %lld of the row dimension exceeds 256 MiB", who, what,
                     (long long)strides[2]);
     return TT_NORM_OK;

@@ -358,7 +358,7 @@ class _AdaLNZeroBase(nn.Module):
     n_chunks = 0
 
     def __init__(self, embedding_dim: int, norm_type: str, bias: bool, fused_kernels: bool,
-                 linear_parallel: bool, config):
+                 linear_parallel: bool, config, fused_eps: Optional[float] = None):
         super().__init__()
         self.silu = nn.SiLU()
         self.linear_parallel = linear_parallel
@@ -369,10 +369,12 @@ class _AdaLNZeroBase(nn.Module):
             if not cols_supported(embedding_dim, torch.float32):  # the strictest element size
                 raise ValueError(f"fused_kernels=True: {_unsupported(embedding_dim, torch.float32)}")
             _require_extension(fused_adaln, "fused_adaln")
-            # the fused kernel stands in for the eager norm the constructor would otherwise build, with that
-            # norm's eps: 1e-6 for nn.LayerNorm as built below, nn.LayerNorm's default 1e-5 for FP32LayerNorm
-            # (the reference's fused branch always passes 1e-6, dit_fusedlayers.py:194-195)
-            self.adaLN = AdaLNCustom(embedding_dim, eps=1e-5 if norm_type == "fp32_layer_norm" else 1e-6)
+            # As in the reference, the fused branch normalises with eps 1e-6 whatever norm_type says
+            # (dit_fusedlayers.py:194-195, 249-250), so a checkpoint trained through the reference's fused branch
+            # sees the same function here.  The eager branch of norm_type="fp32_layer_norm" builds FP32LayerNorm
+            # with nn.LayerNorm's default 1e-5: pass fused_eps=1e-5 to have the fused branch match THAT instead
+            # (the two differ visibly only on rows whose variance is not far above 1e-5).
+            self.adaLN = AdaLNCustom(embedding_dim, eps=1e-6 if fused_eps is None else float(fused_eps))
         elif norm_type == "layer_norm":
             self.norm = nn.LayerNorm(embedding_dim, elementwise_affine=False, eps=1e-6)
         elif norm_type == "fp32_layer_norm":
@@ -394,8 +396,8 @@ class FusedAdaLayerNormZero(_AdaLNZeroBase):
     n_chunks = 6
 
     def __init__(self, embedding_dim: int, num_embeddings: Optional[int] = None, norm_type="layer_norm",
-                 bias=True, fused_kernels=False, linear_parallel=True, config=None):
-        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config)
+                 bias=True, fused_kernels=False, linear_parallel=True, config=None, fused_eps: Optional[float] = None):
+        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config, fused_eps)
         self.emb = None
         if num_embeddings is not None:
             try:
@@ -419,8 +421,8 @@ class FusedAdaLayerNormZeroSingle(_AdaLNZeroBase):
     n_chunks = 3
 
     def __init__(self, embedding_dim: int, norm_type="layer_norm", bias=True, fused_kernels=False,
-                 linear_parallel=True, config=None):
-        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config)
+                 linear_parallel=True, config=None, fused_eps: Optional[float] = None):
+        super().__init__(embedding_dim, norm_type, bias, fused_kernels, linear_parallel, config, fused_eps)
 
     def forward(self, x, emb=None):
         emb = _gather_modulation(self.linear(self.silu(emb)), self.linear_parallel)
@@ -624,8 +626,9 @@ def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSN
     transposes and the two per-head RMSNorms of dit_attention.py:149-214 in one call, and with
     rotary=(freqs_cos, freqs_sin) also the rotary embedding of query and key that follows them
     (dit_attention.py:266-273; tables of S_img <= S rows rotate the first S_img tokens, :435-443).
-    Fused when FUSED_KERNELS is on and the head dimension is one the tuned kernels take (128 for the
-    rotary form); the reference's own sequence of operations otherwise."""
+    Fused when FUSED_KERNELS is on and the kernels take the head dimension; the rotation itself is fused at
+    head dimension 128 and applied as PyTorch ops to the fused norm's output at any other one.  The
+    reference's own sequence of operations otherwise."""
     D = mixed_qkv.shape[-1] // 3
     fusable = (fused_kernels_requested() and mixed_qkv.dtype in _ELEM_BYTES and cols_supported(D, mixed_qkv.dtype)
                and q_norm.eps == k_norm.eps)
@@ -633,8 +636,11 @@ def split_qkv_and_norm(mixed_qkv: torch.Tensor, q_norm: "RMSNorm", k_norm: "RMSN
         return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
     if fusable and D == 128:
         return QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps, *rotary)
-    query, key, value = torch.split(mixed_qkv, [D, D, D], dim=3)
-    query, key, value = q_norm(query.transpose(1, 2)), k_norm(key.transpose(1, 2)), value.transpose(1, 2)
+    if fusable:   # the strided-norm fusion is kept; only the rotation runs as separate ops
+        query, key, value = QKVSplitNormFunction.apply(mixed_qkv, q_norm.weight, k_norm.weight, q_norm.eps)
+    else:
+        query, key, value = torch.split(mixed_qkv, [D, D, D], dim=3)
+        query, key, value = q_norm(query.transpose(1, 2)), k_norm(key.transpose(1, 2)), value.transpose(1, 2)
     if rotary is not None:
         n = rotary[0].shape[0]
         query = torch.cat([rotate_pairs_eager(query[:, :, :n], *rotary), query[:, :, n:]], dim=2)

@@ -24,7 +24,7 @@ import sys
 import time
 
 from teletron_amd.build import ROOT
-from teletron_amd.profile_summary import CACHED_VARIANTS, PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WORKLOAD_INFO
+from teletron_amd.profile_summary import CACHED_VARIANTS, CFG4_PASSES, PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WORKLOAD_INFO
 
 BENCH = ["python3", "bench.py"]
 QUICK = ["--steps", "3", "--warmup", "1", "--no-cpu-baseline"]
@@ -61,8 +61,8 @@ def cfg4(directory, only):
     trace(directory, "trace", ["--steps", "30", "--warmup", "5", "--no-cpu-baseline"])
     pmc(directory, "fetch", "FETCH_SIZE", QUICK)
     pmc(directory, "write", "WRITE_SIZE", QUICK)
-    for p, counters in PASS_COUNTERS.items():
-        pmc(directory, p, counters, QUICK)
+    for p in CFG4_PASSES:
+        pmc(directory, p, PASS_COUNTERS[p], QUICK)
 
 
 def workloads(directory, only):

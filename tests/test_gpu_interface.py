@@ -515,17 +515,27 @@ def test_fp32_layer_norm_variant_is_the_same_kernel_at_eps_1e5(FL, gpu_device, d
 
 @pytest.mark.parametrize("cls_name", ["FusedAdaLayerNormZero", "FusedAdaLayerNormZeroSingle"])
 def test_adaln_zero_fp32_layer_norm_fused_vs_eager_branch(FL, gpu_device, cls_name):
-    """The modules built with norm_type="fp32_layer_norm": the fused branch stands in for FP32LayerNorm
-    (eps 1e-5) and must agree with the eager branch, forward and backward, on small-variance rows where the
-    eps is visible."""
+    """The modules built with norm_type="fp32_layer_norm".  Two choices of eps exist for the fused branch and
+    both are pinned here on small-variance rows, where the eps is visible: the default is the reference's
+    fused branch (eps 1e-6 whatever the norm type, dit_fusedlayers.py:194-195, 249-250: what a checkpoint
+    trained through that branch expects); fused_eps=1e-5 matches the module's own eager branch (FP32LayerNorm
+    with nn.LayerNorm's default eps), forward and backward."""
     torch.manual_seed(3)
     B, S, C = 2, 130, 3072
     cls = getattr(FL, cls_name)
     x = (0.02 * torch.randn(B, S, C, device=gpu_device)).bfloat16()
     temb = torch.randn(B, C, device=gpu_device).bfloat16()
     g = torch.randn(B, S, C, device=gpu_device).bfloat16()
-    fused = cls(C, norm_type="fp32_layer_norm", fused_kernels=True, linear_parallel=False).to(gpu_device).bfloat16()
+    fused = cls(C, norm_type="fp32_layer_norm", fused_kernels=True, linear_parallel=False, fused_eps=1e-5).to(gpu_device).bfloat16()
     eager = cls(C, norm_type="fp32_layer_norm", fused_kernels=False, linear_parallel=False).to(gpu_device).bfloat16()
+    default = cls(C, norm_type="fp32_layer_norm", fused_kernels=True, linear_parallel=False).to(gpu_device).bfloat16()
+    plain = cls(C, norm_type="layer_norm", fused_kernels=False, linear_parallel=False).to(gpu_device).bfloat16()
+    assert default.adaLN.eps == 1e-6 and fused.adaLN.eps == 1e-5
+    default.load_state_dict(fused.state_dict())
+    plain.load_state_dict(fused.state_dict())
+    # default fused branch == the reference's fused branch == LayerNorm at eps 1e-6, and visibly not eps 1e-5
+    yd, yp = default(x, emb=temb)[0], plain(x, emb=temb)[0]
+    assert O.compare_bf16_ulp(yd.detach().cpu(), yp.detach().cpu()).frac_exact > 0.999
     eager.load_state_dict(fused.state_dict())
     xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
     ya, yb = fused(xa, emb=temb), eager(xb, emb=temb)
@@ -533,6 +543,7 @@ def test_adaln_zero_fp32_layer_norm_fused_vs_eager_branch(FL, gpu_device, cls_na
     yb[0].backward(g)
     rep = O.compare_bf16_ulp(ya[0].detach().cpu(), yb[0].detach().cpu())
     assert rep.frac_exact > 0.999, rep
+    assert O.compare_bf16_ulp(yd.detach().cpu(), yb[0].detach().cpu()).frac_exact < 0.9     # 1e-6 vs 1e-5 is visible here
     assert O.frac_outside(ya[0].detach().cpu(), yb[0].detach().cpu(), 1e-2, 1e-3) < 1e-5
     assert O.frac_outside(xa.grad.cpu(), xb.grad.cpu(), 1e-2, 1e-3) < 1e-4
     ga, gb = fused.linear.weight.grad.float().cpu(), eager.linear.weight.grad.float().cpu()
@@ -632,3 +643,38 @@ def test_qkv_split_norm_function_with_rotary_tables(FL, gpu_device, n_txt, monke
     eq, ek, ev = FL.split_qkv_and_norm(mixed.to(gpu_device), qn, kn, rotary=(cos.to(gpu_device), sin.to(gpu_device)))
     assert O.frac_outside(eq.detach().cpu(), q.detach(), 1e-2, 1e-2) == 0.0
     assert O.frac_outside(ek.detach().cpu(), k.detach(), 1e-2, 1e-2) == 0.0
+
+
+def test_split_qkv_and_norm_with_rotary_at_another_head_dimension(FL, gpu_device, monkeypatch):
+    """Head dimension 64 with rotary tables: the rotation is fused for 128 only, but the strided QK-norm is kept
+    (QKVSplitNormFunction without tables, then the rotation as PyTorch ops on its output) instead of falling
+    all the way back to split + contiguous copy + dense norm.  Same results as the eager sequence."""
+    B, S, H, D, n_txt = 2, 77, 5, 64, 9
+    gen = torch.Generator().manual_seed(41)
+    mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()
+    wq = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    wk = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+    gq, gk, gv = (torch.randn(B, H, S, D, generator=gen).bfloat16() for _ in range(3))
+    cos, sin = O.make_rope_tables(S - n_txt, D, seed=5)
+    mc, wqc, wkc = (t.clone().requires_grad_(True) for t in (mixed, wq, wk))
+    q, k, v = torch.split(mc, [D, D, D], dim=3)
+    q = O.eager_qk_norm_rope(q.transpose(1, 2), wqc, cos, sin)
+    k = O.eager_qk_norm_rope(k.transpose(1, 2), wkc, cos, sin)
+    torch.autograd.backward([q, k, v.transpose(1, 2)], [gq, gk, gv])
+    monkeypatch.setenv("FUSED_KERNELS", "1")
+    mg = mixed.to(gpu_device).requires_grad_(True)
+    qn, kn = FL.RMSNorm(D).to(gpu_device).bfloat16(), FL.RMSNorm(D).to(gpu_device).bfloat16()
+    with torch.no_grad():
+        qn.weight.copy_(wq)
+        kn.weight.copy_(wk)
+    calls = []
+    real_apply = FL.QKVSplitNormFunction.apply
+    monkeypatch.setattr(FL.QKVSplitNormFunction, "apply", staticmethod(lambda *a: (calls.append(len(a)), real_apply(*a))[1]))
+    fq, fk, fv = FL.split_qkv_and_norm(mg, qn, kn, rotary=(cos.to(gpu_device), sin.to(gpu_device)))
+    assert calls == [4]                      # the fused strided norm ran, without tables
+    torch.autograd.backward([fq, fk, fv], [t.to(gpu_device) for t in (gq, gk, gv)])
+    yq = O.eager_rmsnorm(mixed[..., :D].transpose(1, 2), wq)
+    fwd_ok(fq, q.detach(), O.rope_excuse(yq, q.detach()))
+    grad_ok(mg.grad, mc.grad, allow=1e-5)
+    grad_ok(qn.weight.grad, wqc.grad)
+    grad_ok(kn.weight.grad, wkc.grad)

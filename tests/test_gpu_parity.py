@@ -254,6 +254,18 @@ def test_full_size_adaln_properties(capi, gpu_device):
     # dshift = column sums of the upstream gradient
     want_dh = grad.float().sum(1)
     assert O.frac_outside(dh.cpu(), want_dh.cpu(), 1e-2, 1e-3) == 0.0
+    # dscale against an independent fp32 column reduction (torch ops) of rnd(g * rnd(xhat)), xhat from the
+    # statistics the forward wrote
+    # (summed in float64: over 118 800 terms an fp32 reduction of its own carries ~1e-3 of rounding); the plain
+    # gradient bar on all but 1e-3 of the columns, and every column within 1e-2 |want| + 2^-8 of its L2 mass
+    xn = ((x.float() - mean.view(1, rows, 1)) * rstd.view(1, rows, 1)).bfloat16()
+    terms = grad * xn
+    del xn
+    want_ds = terms.double().sum(1)
+    l2 = terms.float().pow(2).sum(1).sqrt().double()
+    del terms
+    assert O.frac_outside(ds.cpu(), want_ds.cpu(), 1e-2, 1e-3) <= 1e-3
+    assert bool(((ds.double() - want_ds).abs() <= 1e-2 * want_ds.abs() + 2.0 ** -8 * l2).all())
     # the input's other gradient added inside the kernel == plain backward, then the addition
     other = (0.5 * torch.randn(1, rows, C, device=gpu_device, generator=gen)).bfloat16()
     dxr, dsr, dhr = capi.adaln_backward_residual(grad, other, x, scale, mean, rstd)
