@@ -60,15 +60,14 @@ def _record(case, name, kernel, dev_eager, cpu_eager, truth):
     return rec
 
 
-def _column_sum_bar(case, name, rec, got, want, terms, truth_ok=True):
+def _column_sum_bar(case, name, rec, got, want, terms, plain_allow=1e-3):
     """The bar for dscale / dweight stated at the top; terms [.., rows, C] are the summed products."""
     rows_dim = terms.dim() - 2
     l2 = terms.float().pow(2).sum(rows_dim).sqrt().double().reshape(want.shape)
     g, w = got.double().reshape(want.shape), want.double()
-    assert rec["kernel_vs_device_eager_outside"] <= 1e-3, (case, name, rec)
+    assert rec["kernel_vs_device_eager_outside"] <= plain_allow, (case, name, rec)
     assert bool(((g - w).abs() <= 1e-2 * w.abs() + 2.0 ** -8 * l2).all()), (case, name, rec)
-    if truth_ok:
-        assert rec["kernel_rms"] <= 1.05 * rec["device_eager_rms"] + 1e-30, (case, name, rec)
+    assert rec["kernel_rms"] <= 1.05 * rec["device_eager_rms"] + 1e-30, (case, name, rec)
 
 
 def _stress_rows(B, S, C, dtype, kind, seed):
@@ -103,7 +102,10 @@ def test_adaln_stress_rows_against_device_eager(capi, gpu_device, C, dtype, kind
     assert recs["dx"]["kernel_vs_device_eager_outside"] <= 1e-4, (case, recs["dx"])
     assert recs["dshift"]["kernel_vs_device_eager_outside"] == 0.0, (case, recs["dshift"])
     xn = torch.nn.functional.layer_norm(g["x"], (C,), None, None, EPS)
-    _column_sum_bar(case, "dscale", recs["dscale"], ds, want[2], g["grad"] * xn)
+    # mean 30 sigma: about one xhat in a thousand rounds the other way between two correct fp32 forms (see the top),
+    # which touches every second column sum of 515 rows by an ulp of one term; where the sum itself is small that
+    # exceeds the plain bar (device eager and CPU eager differ from each other on the same 1 % of columns)
+    _column_sum_bar(case, "dscale", recs["dscale"], ds, want[2], g["grad"] * xn, plain_allow=2e-2 if kind == "mean" else 1e-3)
     if dtype == torch.bfloat16:
         rep = O.compare_bf16_ulp(out.cpu(), want[0].cpu(),
                                  excuse_abs=O.adaln_excuse(d["x"], d["scale"], d["shift"], want[0].cpu()))
