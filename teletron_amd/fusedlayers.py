@@ -85,6 +85,15 @@ def fused_kernels_requested() -> bool:
     return bool(int(flag)) if flag else False
 
 
+def eager_fallback_enabled() -> bool:
+    """TELETRON_AMD_FALLBACK=eager restores the reference's silent gating (dit_fusedlayers.py:194-204, 364-370):
+    where the fused path cannot run -- extension not importable, tensor not on a GPU, a row the kernels do
+    not take, a weight whose dtype differs from the input's -- the modules compute the eager formula
+    instead of raising.  Off by default: a training run that asked for fused kernels and silently did not
+    get them is the failure this package would rather report."""
+    return os.environ.get("TELETRON_AMD_FALLBACK", "").strip().lower() == "eager"
+
+
 def _require_extension(mod, name: str):
     if mod is None:
         raise RuntimeError(f"{name} extension is not built/importable ({_IMPORT_ERROR}); "
@@ -365,6 +374,10 @@ class _AdaLNZeroBase(nn.Module):
         self.linear = _make_modulation_linear(embedding_dim, self.n_chunks, bias, linear_parallel, config)
         self.fused_kernels = bool(fused_kernels)
         self.embedding_dim = embedding_dim
+        self.norm_eps = 1e-5 if norm_type == "fp32_layer_norm" else 1e-6   # of the eager norm built below
+        if self.fused_kernels and eager_fallback_enabled() and (
+                fused_adaln is None or not cols_supported(embedding_dim, torch.float32)):
+            self.fused_kernels = False      # the reference's constructor gate: fall through to the eager norm
         if self.fused_kernels:
             if not cols_supported(embedding_dim, torch.float32):  # the strictest element size
                 raise ValueError(f"fused_kernels=True: {_unsupported(embedding_dim, torch.float32)}")
@@ -385,6 +398,9 @@ class _AdaLNZeroBase(nn.Module):
 
     def _modulate(self, x, scale, shift):
         if self.fused_kernels:
+            if eager_fallback_enabled() and not (x.is_cuda and x.dtype in _ELEM_BYTES):
+                xn = F.layer_norm(x, (self.embedding_dim,), None, None, self.adaLN.eps)
+                return xn * (1 + scale[:, None]) + shift[:, None]
             return self.adaLN(x, scale, shift)
         return self.norm(x) * (1 + scale[:, None]) + shift[:, None]
 
@@ -516,7 +532,9 @@ class RMSNorm(nn.Module):
 
     def forward(self, x):
         if fused_kernels_requested() and cols_supported(self.hidden_size, x.dtype):
-            return RMSNormModelFunction.apply(x, self.weight, self.eps, self.hidden_size)
+            if not (eager_fallback_enabled() and (fused_rmsnorm is None or not x.is_cuda
+                                                  or self.weight.dtype != x.dtype)):
+                return RMSNormModelFunction.apply(x, self.weight, self.eps, self.hidden_size)
         return self._norm(x.float()).type_as(x) * self.weight
 
 

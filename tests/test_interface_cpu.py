@@ -233,3 +233,35 @@ def test_c_abi_accepts_zero_rows_without_a_gpu_launch():
     assert L.tt_adaln_forward(None, None, None, None, None, None, 3, 0, 3072, 1e-6, 0, None) == 0
     assert L.tt_rmsnorm_forward(None, None, None, None, -1, 3072, 1e-6, 0, None) == 1
     assert L.tt_rmsnorm_backward_workspace_bytes(0, 3072, 0) == 0
+
+
+def test_eager_fallback_switch_restores_the_reference_gating(monkeypatch):
+    """TELETRON_AMD_FALLBACK=eager: with FUSED_KERNELS on, a tensor the fused path cannot take (here: on the CPU;
+    also a weight of another dtype, or a missing extension) is computed by the eager formula, silently, as
+    the reference does (dit_fusedlayers.py:194-204, 364-370).  Without the switch the same call raises."""
+    from teletron_amd import fusedlayers as FL
+    monkeypatch.setenv("FUSED_KERNELS", "1")
+    monkeypatch.delenv("TELETRON_AMD_FALLBACK", raising=False)
+    x = torch.randn(3, 5, 128).bfloat16()
+    norm = FL.RMSNorm(128).bfloat16()
+    with pytest.raises(ValueError, match="GPU tensor"):
+        norm(x)
+    ada = FL.FusedAdaLayerNormZeroSingle(256, fused_kernels=True, linear_parallel=False)
+    h, temb = torch.randn(2, 7, 256), torch.randn(2, 256)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        ada(h, emb=temb)
+    monkeypatch.setenv("TELETRON_AMD_FALLBACK", "eager")
+    assert FL.eager_fallback_enabled()
+    assert torch.equal(norm(x), O.eager_rmsnorm(x, norm.weight))
+    out, gate = ada(h, emb=temb)
+    c = ada.linear(torch.nn.functional.silu(temb)).chunk(3, dim=1)
+    torch.testing.assert_close(out, O.eager_adaln(h, c[1], c[0]))
+    # an fp32 weight with a bf16 input: eager promotes to fp32, and so does the fallback
+    mixed = FL.RMSNorm(128)
+    assert mixed(x).dtype == torch.float32
+    # the constructor gate: a width the kernels do not take builds the eager norm instead of raising
+    odd = FL.FusedAdaLayerNormZero(66, fused_kernels=True, linear_parallel=False)
+    assert odd.fused_kernels is False and isinstance(odd.norm, torch.nn.LayerNorm)
+    monkeypatch.setenv("TELETRON_AMD_FALLBACK", "")
+    with pytest.raises(ValueError, match="unsupported cols 66"):
+        FL.FusedAdaLayerNormZero(66, fused_kernels=True, linear_parallel=False)
