@@ -32,7 +32,7 @@ ARCH = "gfx950"
 # compiler narrows fp16 chains to half arithmetic and then fuses across a rounding point.
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
              "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip"]
+KERNEL_SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip", "widerow.hip"]
 EXT_MODULES = {"fused_rmsnorm": "fused_rmsnorm_ext.cpp", "fused_adaln": "fused_adaln_ext.cpp"}
 
 

@@ -26,6 +26,11 @@
 #ifndef TTN_ANY_BWD_STORE
 #define TTN_ANY_BWD_STORE 1
 #endif
+// 1: dense rows of more than 384 pieces go to the kernels of widerow.hip (four wavefronts per row); 0: they stay
+// with the one-wavefront-per-row kernels here (8, 12 or 16 accesses per lane), which strided views always use.
+#ifndef TTN_WIDE_ROWS
+#define TTN_WIDE_ROWS 1
+#endif
 
 namespace ttn {
 
@@ -694,6 +699,7 @@ static int rmsnorm_forward_on(void *out, float *rstd, const void *x, const void 
 
 int anywidth_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
                              double eps, int dtype, hipStream_t stream) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype)) return widerow_rmsnorm_forward(out, rstd, x, w, rows, cols, eps, dtype, stream);
     return rmsnorm_forward_on(out, rstd, x, w, DenseRows{rows}, rows, cols, eps, dtype, stream);
 }
 
@@ -706,7 +712,13 @@ static size_t backward_scratch(int64_t batch, int64_t rows_per_sample, int64_t c
     if (batch <= 0 || rows_per_sample <= 0 || !anywidth_supported(cols, dtype)) return 0;
     RowPlan p;
     if (plan_for(&p, batch, rows_per_sample, geometry_for(cols, dtype), true) != TT_NORM_OK) return 0;
-    return (size_t)p.blocks * nsets * cols * sizeof(float);
+    size_t need = (size_t)p.blocks * nsets * cols * sizeof(float);
+    if (TTN_WIDE_ROWS && nsets <= 2 && widerow_takes(cols, dtype)) {  // dense rows take the other kernels, strided views these
+        const size_t wide = widerow_backward_workspace_bytes(batch, rows_per_sample, cols, dtype, nsets);
+        if (wide == 0) return 0;
+        if (wide > need) need = wide;
+    }
+    return need;
 }
 
 size_t anywidth_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
@@ -736,6 +748,8 @@ static int rmsnorm_backward_on(void *dx, void *dw, const void *g, const void *x,
 int anywidth_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w,
                               const float *rstd, int64_t rows, int64_t cols, int dtype, void *ws,
                               size_t ws_bytes, hipStream_t stream) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_rmsnorm_backward(dx, dw, g, x, w, rstd, rows, cols, dtype, ws, ws_bytes, stream);
     return rmsnorm_backward_on(dx, dw, g, x, w, rstd, DenseRows{rows}, rows, cols, dtype, ws, ws_bytes, stream);
 }
 
@@ -772,6 +786,9 @@ static int adaln_forward_any(void *out, float *mean, float *rstd, const void *x,
 int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale,
                            const void *shift, int64_t batch, int64_t rows_per_sample, int64_t cols, double eps,
                            int dtype, hipStream_t stream, bool seq_first) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_adaln_forward(out, mean, rstd, x, scale, shift, batch, rows_per_sample, cols, eps, dtype, seq_first,
+                                     stream);
     return adaln_forward_any<false>(out, mean, rstd, x, scale, shift, AdalnExtra{nullptr, nullptr, nullptr, nullptr},
                                     batch, rows_per_sample, cols, eps, dtype, seq_first, stream);
 }
@@ -815,6 +832,9 @@ int anywidth_adaln_backward(void *dx, void *dscale, void *dshift, const void *g,
                             const void *scale, const float *mean, const float *rstd, int64_t batch,
                             int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
                             hipStream_t stream, bool seq_first) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_adaln_backward(dx, dscale, dshift, g, x, scale, mean, rstd, batch, rows_per_sample, cols, dtype, ws,
+                                      ws_bytes, seq_first, stream);
     return adaln_backward_any<false, false>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
                                             AdalnExtra{nullptr, nullptr, nullptr, nullptr}, batch, rows_per_sample, cols,
                                             dtype, ws, ws_bytes, seq_first, stream);

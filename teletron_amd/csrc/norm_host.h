@@ -111,4 +111,19 @@ int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const
                                      int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
                                      size_t ws_bytes, hipStream_t stream);
 
+// ---- wide rows (widerow.hip): more than 384 16-byte pieces per row, four wavefronts per row -----
+// Dense rows only (contiguous, or sample-major / sequence-first AdaLN); same argument meaning as above.
+bool widerow_takes(int64_t cols, int dtype);
+size_t widerow_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, int nsets);
+int widerow_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
+                            double eps, int dtype, hipStream_t stream);
+int widerow_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, const void *w, const float *rstd,
+                             int64_t rows, int64_t cols, int dtype, void *ws, size_t ws_bytes, hipStream_t stream);
+int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale, const void *shift,
+                          int64_t batch, int64_t rows_per_sample, int64_t cols, double eps, int dtype, bool seq_first,
+                          hipStream_t stream);
+int widerow_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x, const void *scale,
+                           const float *mean, const float *rstd, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                           int dtype, void *ws, size_t ws_bytes, bool seq_first, hipStream_t stream);
+
 }  // namespace ttn

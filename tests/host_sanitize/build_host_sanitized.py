@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "teletron_amd", "csrc")
-SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip", "probe.hip"]
+SOURCES = ["norm_host.hip", "rmsnorm.hip", "adaln.hip", "anywidth.hip", "widerow.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 SAN = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-Xarch_host",
        "-fno-sanitize-recover=undefined", "-Xarch_host", "-fno-omit-frame-pointer"]
