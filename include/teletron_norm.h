@@ -226,12 +226,12 @@ int tt_adaln_backward_seq_first(void *dx, void *dscale, void *dshift, const void
  * TT_NORM_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
  * ends); the call allocates and frees nothing.  Shapes whose scratch need
  * (tt_adaln_backward_workspace_bytes) exceeds the array return TT_NORM_EWORKSPACE: at 3072
- * columns that is batch > 682; every supported width fits for batch <= 256.  Results are
+ * columns that is batch > 1365; every supported width fits for batch <= 256.  Results are
  * bit-identical to tt_adaln_backward.  All calls on one GPU share that GPU's array: calls that
  * overlap in time on one GPU (different streams or threads) race; on one stream they are safe.
  * The array used is the CURRENT device's (hipGetDevice), which must be the device that holds the
  * tensors: a dx that lives on another device is refused with TT_NORM_EINVAL. */
-#define TT_NORM_STATIC_SCRATCH_BYTES (16u << 20)
+#define TT_NORM_STATIC_SCRATCH_BYTES (32u << 20)
 int tt_adaln_backward_static(void *dx, void *dscale, void *dshift, const void *dout, const void *x,
                              const void *scale, const float *mean, const float *rstd,
                              int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype,

@@ -727,7 +727,8 @@ int tt_adaln_forward_xnorm(void *out, void *x_norm, float *rstd, const void *x, 
 
 size_t tt_adaln_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype) {
     if (batch <= 0 || rows_per_sample <= 0 || !tt_norm_supported(cols, dtype)) return 0;
-    if (!tuned_shape(cols, dtype)) return anywidth_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype);
+    if (!tuned_shape(cols, dtype) || dense_backward_on_wide_rows(cols, dtype))
+        return anywidth_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return 0;
@@ -745,7 +746,7 @@ int tt_adaln_backward(void *dx, void *dscale, void *dshift, const void *dout, co
     if (st != TT_NORM_OK) return st;
     if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward: null dscale/dshift/mean/rstd");
-    if (!tuned_shape(cols, dtype))
+    if (!tuned_shape(cols, dtype) || dense_backward_on_wide_rows(cols, dtype))
         return anywidth_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols,
                                        dtype, workspace, workspace_bytes, (hipStream_t)stream);
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream};
@@ -800,7 +801,7 @@ int tt_adaln_backward_seq_first(void *dx, void *dscale, void *dshift, const void
     if (st != TT_NORM_OK) return st;
     if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward_seq_first: null dscale/dshift/mean/rstd");
-    if (!tuned_shape(cols, dtype))
+    if (!tuned_shape(cols, dtype) || dense_backward_on_wide_rows(cols, dtype))
         return anywidth_adaln_backward(dx, dscale, dshift, dout, x, scale, mean, rstd, batch, rows_per_sample, cols,
                                        dtype, workspace, workspace_bytes, (hipStream_t)stream, true);
     const AdalnArgs a{batch, rows_per_sample, 0.0, (hipStream_t)stream, true};

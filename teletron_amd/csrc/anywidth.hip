@@ -26,11 +26,6 @@
 #ifndef TTN_ANY_BWD_STORE
 #define TTN_ANY_BWD_STORE 1
 #endif
-// 1: dense rows of more than 384 pieces go to the kernels of widerow.hip (four wavefronts per row); 0: they stay
-// with the one-wavefront-per-row kernels here (8, 12 or 16 accesses per lane), which strided views always use.
-#ifndef TTN_WIDE_ROWS
-#define TTN_WIDE_ROWS 1
-#endif
 
 namespace ttn {
 

@@ -111,9 +111,18 @@ int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const
                                      int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
                                      size_t ws_bytes, hipStream_t stream);
 
+// 1: dense rows of more than 384 pieces go to the kernels of widerow.hip (four wavefronts per row); 0: they stay
+// with the one-wavefront-per-row kernels of anywidth.hip (8, 12 or 16 accesses per lane), which strided views always use.
+#ifndef TTN_WIDE_ROWS
+#define TTN_WIDE_ROWS 1
+#endif
+
 // ---- wide rows (widerow.hip): more than 384 16-byte pieces per row, four wavefronts per row -----
 // Dense rows only (contiguous, or sample-major / sequence-first AdaLN); same argument meaning as above.
 bool widerow_takes(int64_t cols, int dtype);
+// Dense backward calls at a tuned width that run on the wide-row kernels all the same (fp32 rows of 3072 columns: a
+// wavefront that owns such a row has registers for one row buffer only).
+bool dense_backward_on_wide_rows(int64_t cols, int dtype);
 size_t widerow_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, int nsets);
 int widerow_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
                             double eps, int dtype, hipStream_t stream);

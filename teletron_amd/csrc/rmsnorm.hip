@@ -633,7 +633,8 @@ int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight
 
 size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype) {
     if (rows <= 0 || !tt_norm_supported(cols, dtype)) return 0;
-    if (!tuned_shape(cols, dtype)) return anywidth_rmsnorm_backward_workspace_bytes(rows, cols, dtype);
+    if (!tuned_shape(cols, dtype) || dense_backward_on_wide_rows(cols, dtype))
+        return anywidth_rmsnorm_backward_workspace_bytes(rows, cols, dtype);
     int st = TT_NORM_OK;
     const int cus = current_device_cus(&st);
     if (st != TT_NORM_OK) return 0;
@@ -648,7 +649,7 @@ int tt_rmsnorm_backward(void *dx, void *dweight, const void *dout, const void *x
     int st = check_rms_args("tt_rmsnorm_backward", rows, cols, dtype, {dx, dout, x, weight});
     if (st != TT_NORM_OK) return st;
     if (!dweight || (!rstd && rows > 0)) return fail(TT_NORM_EINVAL, "tt_rmsnorm_backward: null dweight/rstd");
-    if (!tuned_shape(cols, dtype))
+    if (!tuned_shape(cols, dtype) || dense_backward_on_wide_rows(cols, dtype))
         return anywidth_rmsnorm_backward(dx, dweight, dout, x, weight, rstd, rows, cols, dtype, workspace,
                                          workspace_bytes, (hipStream_t)stream);
 #define CALL(T, C)                                                                                  \

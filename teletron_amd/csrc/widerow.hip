@@ -642,6 +642,13 @@ bool widerow_takes(int64_t cols, int dtype) {
     return cols / (16 / (int64_t)elem_bytes(dtype)) >= kWidePiecesMin;
 }
 
+#ifndef TTN_F32_3072_BWD_WIDE
+#define TTN_F32_3072_BWD_WIDE 1
+#endif
+bool dense_backward_on_wide_rows(int64_t cols, int dtype) {
+    return TTN_F32_3072_BWD_WIDE && TTN_WIDE_ROWS && dtype == TT_NORM_F32 && cols == 3072;
+}
+
 // pieces per wavefront (a quarter of the row, rounded up) and the accesses per lane that takes
 static int wide_pieces_per_wave(int64_t cols, int dtype) {
     const int64_t pieces = cols / (16 / (int64_t)elem_bytes(dtype));

@@ -215,7 +215,13 @@ def test_strided_writes_stay_inside_their_slices(capi, gpu_device, dtype, B, S, 
         assert torch.equal(dmixed[~written], fill[~written]), f"slice {i}: wrote outside its slice of the gradient"
         out2, rstd2 = capi.rmsnorm_forward(view.contiguous(), w, EPS)
         dx2, dw2 = capi.rmsnorm_backward(grads[i], view.contiguous(), w, rstd2)
-        assert torch.equal(outs[i], out2) and torch.equal(rstds[i], rstd2) and torch.equal(dview.contiguous(), dx2)
+        assert torch.equal(outs[i], out2) and torch.equal(rstds[i], rstd2)
+        if D * mixed.element_size() // 16 > 384:
+            # dense rows of more than 384 pieces run their backward on other kernels (four wavefronts per row) than
+            # a strided view does: the row sums are formed in another order
+            torch.testing.assert_close(dview.contiguous(), dx2, rtol=1e-5, atol=1e-6)
+        else:
+            assert torch.equal(dview.contiguous(), dx2)
     dv = dmixed[..., 2 * D:].transpose(1, 2)
     ds = dv.stride()
     before = dmixed.clone()

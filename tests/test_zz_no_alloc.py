@@ -53,13 +53,16 @@ def test_static_scratch_backward_matches_tt_adaln_backward(gpu_device):
     _both_ways(capi, gpu_device, 1, 37, 3072, torch.bfloat16, seed=12)
     _both_ways(capi, gpu_device, 3, 5, 1536, torch.float16, seed=13)
     _both_ways(capi, gpu_device, 1, 700, 128, torch.float32, seed=14)
+    # rows of more than 384 pieces (four wavefronts per row, two workgroups per compute unit), then fewer of them
+    _both_ways(capi, gpu_device, 2, 1301, 8192, torch.bfloat16, seed=15)
+    _both_ways(capi, gpu_device, 1, 9, 3072, torch.float32, seed=16)
 
 
 def test_static_scratch_backward_rejects_what_does_not_fit(gpu_device):
     from teletron_amd import capi
     L = capi.lib()
-    cols, batch = 3072, 700                      # 700 workgroups x 24 KiB of partial sums > 16 MiB
-    assert L.tt_adaln_backward_workspace_bytes(batch, 4, cols, capi.BF16) > 16 << 20
+    cols, batch = 3072, 1400                     # 1400 workgroups x 24 KiB of partial sums > 32 MiB
+    assert L.tt_adaln_backward_workspace_bytes(batch, 4, cols, capi.BF16) > 32 << 20
     t = torch.zeros(batch * 4 * cols, dtype=torch.bfloat16, device=gpu_device)
     s = torch.zeros(batch * cols, dtype=torch.bfloat16, device=gpu_device)
     f = torch.zeros(batch * 4, dtype=torch.float32, device=gpu_device)
