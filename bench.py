@@ -82,6 +82,10 @@ WORKLOADS = {
     "cached-set": "the four cfg4 kernels on working sets that stay in the 256 MB last-level cache (4096 and 8192 rows x "
                   "3072 bf16, the same buffers launch after launch): what the kernels' own instruction streams "
                   "allow when memory is not the limit, as the per-row slope between the two sizes",
+    "timeline-cfg3": "cfg3's step (AdaLN forward, backward, column reducer; 29700 x 3072 bf16, three rotating buffer "
+                     "sets, back to back) seen from inside: every wavefront's start and end on the constant 100 MHz "
+                     "clock, from a measurement build of the library (python -m teletron_amd.build --variant LIB "
+                     "--flag=-DTTN_WAVE_CLOCK=1, loaded with TELETRON_AMD_LIB=LIB); --steps = timelines collected",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -437,6 +441,103 @@ def cached_set(args, torch, capi, dev):
     }))
 
 
+def wave_timeline(args, torch, capi, dev):
+    """Where a short step spends its time: the ramp of each kernel (first to last wavefront start), its tail (first
+    to last wavefront end), the gaps between kernels, and in the persistent backward the wavefronts that carry one
+    row more than the others.  Needs the measurement build (see WORKLOADS); figures are medians over the collected
+    timelines, in microseconds from the first wavefront start of the forward kernel."""
+    import numpy as np
+
+    L = capi.lib()
+    try:
+        set_clock, clock_bytes = L.tt_norm_debug_wave_clock, L.tt_norm_debug_wave_clock_bytes
+    except AttributeError:
+        print("timeline-cfg3 needs a library built with -DTTN_WAVE_CLOCK=1 (python -m teletron_amd.build --variant "
+              "LIB.so --flag=-DTTN_WAVE_CLOCK=1; TELETRON_AMD_LIB=LIB.so)", file=sys.stderr)
+        sys.exit(2)
+    set_clock.argtypes, set_clock.restype = [ctypes.c_void_p], ctypes.c_int
+    clock_bytes.argtypes, clock_bytes.restype = [], ctypes.c_size_t
+    sets = [build_workload("cfg3", torch, capi, dev)[0] for _ in range(3)]
+    rows = 29700
+    buf = torch.zeros(clock_bytes() // 8, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    if set_clock(ctypes.c_void_p(buf.data_ptr())) != 0:
+        raise RuntimeError("tt_norm_debug_wave_clock failed")
+    slots = buf.numel() // (3 * 4)
+    kinds = ("adaln_forward", "adaln_backward", "column_reducer")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    collected = []
+    turn = 0
+    for _ in range(max(1, min(args.steps, 25))):
+        buf.zero_()
+        torch.cuda.synchronize()
+        for i in range(args.warmup + 1):      # back to back; the last step's marks are the ones that survive
+            if i == args.warmup:
+                e0.record()
+            turn += 1
+            for _, fn, _ in sets[turn % 3]:
+                fn()
+        e1.record()
+        torch.cuda.synchronize()
+        t = buf.view(3, slots, 4).cpu().numpy().astype(np.float64)
+        rec = {"step_us_by_events": e0.elapsed_time(e1) * 1e3}
+        origin = None
+        for k, name in enumerate(kinds):
+            a = t[k][t[k][:, 0] != 0]
+            if origin is None:
+                origin = a[:, 0].min()
+            st, en = (a[:, 0] - origin) / 100.0, (a[:, 1] - origin) / 100.0     # 100 MHz ticks -> us
+            r = {"wavefronts": int(len(a)), "first_start": st.min(), "last_start": st.max(), "first_end": en.min(),
+                 "last_end": en.max(), "median_wavefront_life": float(np.median(en - st))}
+            lo, hi = st.min(), en.max()
+            r["active_at_tenths"] = [int(((st <= x) & (en > x)).sum()) for x in np.linspace(lo, hi, 11)[:-1] + (hi - lo) / 20]
+            if name == "adaln_backward":
+                done = (a[:, 2] - origin) / 100.0
+                w = np.nonzero(t[k][:, 0] != 0)[0]
+                per_wave = rows // len(a)
+                extra = w < rows - per_wave * len(a)      # these wavefronts own one row more
+                r.update({"rows_per_wavefront": per_wave, "wavefronts_with_one_more": int(extra.sum()),
+                          "rows_done_first": done.min(), "rows_done_median": float(np.median(done)),
+                          "rows_done_last_without_extra": done[~extra].max(),
+                          "rows_done_last_with_extra": done[extra].max() if extra.any() else None,
+                          "us_per_row_median": float(np.median((done - st) / (per_wave + extra)))})
+                if len(a) % 4 == 0:      # per workgroup: its slowest wavefront's last row -> its partial row written
+                    wg_done, wg_end = done.reshape(-1, 4), en.reshape(-1, 4)
+                    r["partial_row_flush_median"] = float(np.median(wg_end.max(axis=1) - wg_done.max(axis=1)))
+                    r["rows_done_spread_inside_workgroup_median"] = float(np.median(wg_done.max(axis=1) - wg_done.min(axis=1)))
+            rec[name] = r
+        rec["gap_forward_to_backward"] = rec["adaln_backward"]["first_start"] - rec["adaln_forward"]["last_end"]
+        rec["gap_backward_to_reducer"] = rec["column_reducer"]["first_start"] - rec["adaln_backward"]["last_end"]
+        rec["span"] = rec["column_reducer"]["last_end"]
+        collected.append(rec)
+
+    def med(path):
+        vals = []
+        for rec in collected:
+            v = rec
+            for key in path:
+                v = v[key]
+            vals.append(v)
+        if vals[0] is None:
+            return None
+        if isinstance(vals[0], list):
+            return [int(np.median([v[i] for v in vals])) for i in range(len(vals[0]))]
+        return round(float(np.median(vals)), 2)
+
+    out = {}
+    for key, v in collected[0].items():
+        out[key] = {k2: med((key, k2)) for k2 in v} if isinstance(v, dict) else med((key,))
+    set_clock(None)
+    step_us = out["step_us_by_events"]
+    algo = 5 * rows * COLS * 2
+    print(json.dumps({
+        "metric": "timeline of cfg3's step from per-wavefront clocks (medians, us)", "value": round(algo / step_us / 1e3, 1),
+        "unit": "GB/s", "n_gpus": 1, "steps": len(collected), "warmup": args.warmup, "ms_per_step": round(step_us / 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": WORKLOADS["timeline-cfg3"], "rows": rows, "cols": COLS}, "timeline_us": out,
+    }))
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -535,6 +636,9 @@ def main():
         return
     if args.workload == "cached-set":
         cached_set(args, torch, capi, dev)
+        return
+    if args.workload == "timeline-cfg3":
+        wave_timeline(args, torch, capi, dev)
         return
     calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)
     headline = args.workload == "cfg4"

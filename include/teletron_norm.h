@@ -97,7 +97,8 @@ int tt_norm_wide_forms_supported(int64_t cols, int dtype);
 int tt_rmsnorm_forward(void *out, float *rstd, const void *x, const void *weight,
                        int64_t rows, int64_t cols, double eps, int dtype, void *stream);
 
-/* Bytes of scratch tt_rmsnorm_backward* need for this shape. */
+/* Bytes of scratch tt_rmsnorm_backward* need for this shape.  Scratch passed to any backward entry point must be
+ * 16-byte aligned (TT_NORM_EALIGN otherwise), like every tensor. */
 size_t tt_rmsnorm_backward_workspace_bytes(int64_t rows, int64_t cols, int dtype);
 
 /* Native backward from the saved input: dx [rows, cols], dweight [cols].

@@ -127,6 +127,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
     const int wave = wave_id_in_block();
     const int64_t b = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
+    wave_clock_mark(kClockAdalnFwd, 0);
 
     // This sample's modulation row, staged once per workgroup through LDS AS FP32: each thread forms
     // t = rnd(1 + scale) for its share of the 16-byte pieces and stores t and shift unpacked, four
@@ -256,6 +257,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(sizeof(T) == 2 
             if (ok) wo.put(k * LANES, E::pack(v));
         }
     }
+    wave_clock_mark(kClockAdalnFwd, 1);
 }
 
 // Backward.  FROM_XNORM = false: xin is the saved input x, statistics mean/rstd.
@@ -292,13 +294,14 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     // A row's first pass starts only when the stores of the row before it have left the wavefront
     // (see the RMSNorm backward): 359 us with this wait, 366 us without, at 118 800 rows.
     constexpr bool kDrainStores = TTN_BWD_DRAIN_STORES && TTN_ADALN_BWD_STORE && !GATED && kRowBuffers == 2 && C >= 1024;
-    __shared__ float lds[NSETS * C];
+    __shared__ __align__(16) float lds[kFlushLdsFloats<NSETS, C>];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
     const int l = lane % LANES;
     const int wave = wave_id_in_block();
     const int64_t smp = blockIdx.x / blocks_per_sample;
     const int slot = blockIdx.x % blocks_per_sample;
+    wave_clock_mark(kClockAdalnBwd, 0);
 
     constexpr bool kPackedProducts = kHasDot2<T> && (TTN_BWD_PACKED_MATH & 1) != 0;
     constexpr bool kPackedColumnSums = kHasDot2<T> && (TTN_BWD_PACKED_MATH & 2) != 0;
@@ -551,8 +554,16 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
         row_pipeline<2, true, RowRegs>(grp, groups, stride, fetch, process);
     else
         row_pipeline<kRowBuffers, TTN_ADALN_BWD_PREFETCH_MID != 0, RowRegs>(grp, groups, stride, fetch, process);
+    wave_clock_mark(kClockAdalnBwd, 2);  // rows done; what follows is the workgroup's partial row
     flush_column_partials<G, NSETS>(acc, partial + (int64_t)blockIdx.x * (NSETS * C), lds);
+    wave_clock_mark(kClockAdalnBwd, 1);
 }
+
+#if TTN_WAVE_CLOCK
+int adaln_set_wave_clock(void *buf) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(ttn_wave_clock_buf), &buf, sizeof(buf)) == hipSuccess ? TT_NORM_OK : TT_NORM_EHIP;
+}
+#endif
 
 // Same launch policy as RMSNorm: forward one-shot at 3072 columns, backward one
 // workgroup per compute unit.
@@ -630,6 +641,7 @@ static int adaln_backward_t(void *dx, void *dscale, void *dshift, const void *g,
     const size_t need = (size_t)p.blocks * NSETS * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
+    if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "adaln backward: workspace %p not 16-byte aligned", ws);
     {
         RowKernelProfile prof(a.stream);
         adaln_bwd_kernel<T, C, FROM_XNORM, GATED, RES><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, a.stream>>>(

@@ -442,6 +442,32 @@ __device__ __forceinline__ int wave_id_in_block() {
     return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }
 
+// Measurement builds only (-DTTN_WAVE_CLOCK=1): every wavefront of an instrumented kernel records the constant
+// 100 MHz clock when it starts and when its last memory operation has completed, into a buffer the host hands
+// over with tt_norm_debug_wave_clock(): entry ((kernel_id * kWaveClockSlots + wavefront) * 4 + which), which = 0
+// start, 1 end, 2 an intermediate point of the kernel's choosing.  The
+// pointer is one variable per translation unit; a null pointer records nothing.  0 in a shipped build: the
+// calls compile to nothing.
+#ifndef TTN_WAVE_CLOCK
+#define TTN_WAVE_CLOCK 0
+#endif
+constexpr int kWaveClockSlots = 1 << 20;
+enum WaveClockKernel { kClockAdalnFwd = 0, kClockAdalnBwd = 1, kClockColReduce = 2, kClockKernels = 3 };
+#if TTN_WAVE_CLOCK
+static __device__ unsigned long long *ttn_wave_clock_buf = nullptr;
+__device__ __forceinline__ void wave_clock_mark(int kernel_id, int which) {
+    unsigned long long *buf = ttn_wave_clock_buf;
+    if (!buf) return;
+    if (which) __builtin_amdgcn_s_waitcnt(0);  // loads and stores of this wavefront have completed
+    const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+    const size_t w = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if ((threadIdx.x & 63) == 0 && w < (size_t)kWaveClockSlots)
+        buf[((size_t)kernel_id * kWaveClockSlots + w) * 4 + which] = t;
+}
+#else
+__device__ __forceinline__ void wave_clock_mark(int, int) {}
+#endif
+
 // Software pipeline over the rows of one wavefront.  `fetch(buf, grp)` issues the
 // loads of a row, `process(buf, mid)` consumes them and calls `mid()` once
 // between its two register passes.  grp advances by `stride` and is
@@ -575,9 +601,22 @@ struct SampleLayout {
     __device__ __forceinline__ int64_t row(int64_t b, int64_t r) const { return b * sample_stride + r * row_stride; }
 };
 
+// How a workgroup folds the column sums of its four wavefronts into its partial row:
+//   1: every wavefront deposits its sums in an LDS region of its own, one barrier, then all threads add the four
+//      regions in wavefront order and write the row in 16-byte pieces (kRowWaves * NSETS * C floats of LDS);
+//   0: wavefront 0 deposits, wavefronts 1.. add in turn into one region (four barriers), 4-byte writes.
+// Both form ((w0 + w1) + w2) + w3 per column: bit-identical.  At 3072 columns and two sets the first takes
+// about 1.5 us less per workgroup, which is time at the end of the kernel that nothing overlaps.
+#ifndef TTN_FLUSH_PARALLEL
+#define TTN_FLUSH_PARALLEL 1
+#endif
+template <int NSETS, int C>
+inline constexpr int kFlushLdsFloats = (TTN_FLUSH_PARALLEL ? kRowWaves : 1) * NSETS * C;
+
 // Adds this workgroup's per-lane column accumulators (acc[k][j] belongs to
 // column (k*LANES + l)*VEC + j) across the rows of each wavefront and across
-// wavefronts in fixed order, and writes one fp32 row of NSETS*C partial sums.
+// wavefronts in fixed order, and writes one fp32 row of NSETS*C partial sums
+// (16-byte aligned).  `lds` holds kFlushLdsFloats<NSETS, C> floats.
 template <typename G, int NSETS>
 __device__ __forceinline__ void flush_column_partials(float (&acc)[NSETS][G::CHUNKS][G::VEC],
                                                       float *__restrict__ partial_row, float *lds) {
@@ -594,6 +633,35 @@ __device__ __forceinline__ void flush_column_partials(float (&acc)[NSETS][G::CHU
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[s][k][j] = fold_rows_of_wave<LANES>(acc[s][k][j]);
 
+#if TTN_FLUSH_PARALLEL
+    static_assert(VEC % 4 == 0 && (NSETS * C) % 4 == 0, "columns come in 16-byte pieces of fp32");
+    if (sub == 0) {
+        u32x4 *mine = reinterpret_cast<u32x4 *>(lds + wave * (NSETS * C));
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s)
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+                for (int q = 0; q < VEC / 4; ++q)
+                    mine[(s * C + (k * LANES + l) * VEC) / 4 + q] =
+                        u32x4{as_u32(acc[s][k][4 * q]), as_u32(acc[s][k][4 * q + 1]), as_u32(acc[s][k][4 * q + 2]),
+                              as_u32(acc[s][k][4 * q + 3])};
+    }
+    __syncthreads();
+    const u32x4 *all = reinterpret_cast<const u32x4 *>(lds);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(partial_row);
+    constexpr int kPieces = NSETS * C / 4;
+    for (int i = threadIdx.x; i < kPieces; i += kRowThreads) {
+        u32x4 sum = all[i];
+#pragma unroll
+        for (int wv = 1; wv < kRowWaves; ++wv) {  // wavefront order: one fixed association
+            const u32x4 v = all[wv * kPieces + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sum[j] = as_u32(as_f32(sum[j]) + as_f32(v[j]));
+        }
+        dst[i] = sum;
+    }
+#else
     // wavefront 0 deposits, wavefronts 1.. add in turn: one fixed order
     for (int wv = 0; wv < kRowWaves; ++wv) {
         if (wave == wv && sub == 0) {
@@ -609,6 +677,7 @@ __device__ __forceinline__ void flush_column_partials(float (&acc)[NSETS][G::CHU
         __syncthreads();
     }
     for (int i = threadIdx.x; i < NSETS * C; i += kRowThreads) partial_row[i] = lds[i];
+#endif
 }
 
 }  // namespace ttn

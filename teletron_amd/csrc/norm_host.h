@@ -117,6 +117,9 @@ int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const
 #define TTN_WIDE_ROWS 1
 #endif
 
+// Measurement builds only (-DTTN_WAVE_CLOCK=1): sets the timestamp buffer of the kernels in adaln.hip.
+int adaln_set_wave_clock(void *buf);
+
 // ---- wide rows (widerow.hip): more than 384 16-byte pieces per row, four wavefronts per row -----
 // Dense rows only (contiguous, or sample-major / sequence-first AdaLN); same argument meaning as above.
 bool widerow_takes(int64_t cols, int dtype);

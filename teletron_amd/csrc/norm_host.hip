@@ -104,6 +104,7 @@ __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
     T *__restrict__ out0, T *__restrict__ out1, T *__restrict__ out2, const float *__restrict__ partial,
     int blocks_per_sample, int C, int ncols, int col_blocks) {
     __shared__ float strands[kRedStrands][kRedCols + 1];
+    wave_clock_mark(kClockColReduce, 0);
     const int tx = threadIdx.x % kRedCols;
     const int ty = threadIdx.x / kRedCols;
     const int64_t b = blockIdx.x / col_blocks;
@@ -131,6 +132,7 @@ __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
         T *dst = col < C ? out0 : (col < 2 * C ? out1 : out2);  // column sets of C columns each
         store_scalar<T>(dst + b * C + col % C, s);
     }
+    wave_clock_mark(kClockColReduce, 1);
 }
 
 int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, int64_t batch,
@@ -173,6 +175,16 @@ const char *tt_norm_status_string(int status) {
 }
 
 const char *tt_norm_last_error(void) { return g_last_error; }
+
+#if TTN_WAVE_CLOCK
+// Measurement builds only: hands the instrumented kernels a device buffer of kClockKernels * kWaveClockSlots * 4
+// 64-bit entries (null switches the recording off).  Synchronous; call it while nothing is running.
+int tt_norm_debug_wave_clock(void *buf) {
+    if (hipMemcpyToSymbol(HIP_SYMBOL(ttn_wave_clock_buf), &buf, sizeof(buf)) != hipSuccess) return TT_NORM_EHIP;
+    return adaln_set_wave_clock(buf);
+}
+size_t tt_norm_debug_wave_clock_bytes(void) { return (size_t)kClockKernels * kWaveClockSlots * 4 * sizeof(unsigned long long); }
+#endif
 
 int tt_norm_supported(int64_t cols, int dtype) {
     return (tuned_shape(cols, dtype) || anywidth_supported(cols, dtype)) ? 1 : 0;

@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kRowThreads) TTN_MIN_WAVES_PER_SIMD(C >= 1024 ? TTN
     // one wavefront never has more than one row of loads plus one row of stores outstanding.  Measured
     // at 118 800 rows: 354 us with this wait, 365 us when the first pass waits for its loads alone.
     constexpr bool kDrainStores = TTN_BWD_DRAIN_STORES && TTN_RMS_BWD_STORE && kRowBuffers == 2 && C >= 1024;
-    __shared__ float lds[C];
+    __shared__ __align__(16) float lds[kFlushLdsFloats<1, C>];
     const int lane = threadIdx.x & 63;
     const int sub = lane / LANES;
     const int l = lane % LANES;
@@ -570,6 +570,7 @@ static int rmsnorm_backward_t(void *dx, void *dw, const void *g, const void *xin
     const size_t need = (size_t)p.blocks * C * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
+    if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "rmsnorm backward: workspace %p not 16-byte aligned", ws);
     {
         RowKernelProfile prof(stream);
         rmsnorm_bwd_kernel<T, C, FROM_OUT, Map, Rope><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(
