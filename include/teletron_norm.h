@@ -43,8 +43,10 @@ extern "C" {
 
 /* 2: adds tt_norm_wide_forms_supported; the gated residual and residual entry points take every row of
  *    up to 384 16-byte pieces (they took 3072 columns only); the measurement kernels tt_norm_stream_copy
- *    and tt_norm_stream_probe left this library for libteletron_probe.so (include/teletron_probe.h). */
-#define TT_NORM_ABI_VERSION 2
+ *    and tt_norm_stream_probe left this library for libteletron_probe.so (include/teletron_probe.h).
+ * 3: the gated residual and residual entry points take every supported row (up to 1024 pieces); scratch passed
+ *    to a backward entry point must be 16-byte aligned; TT_NORM_STATIC_SCRATCH_BYTES is 32 MiB. */
+#define TT_NORM_ABI_VERSION 3
 
 enum tt_norm_status {
     TT_NORM_OK = 0,
@@ -81,9 +83,9 @@ int tt_norm_supported(int64_t cols, int dtype);
 int tt_norm_tuned(int64_t cols, int dtype);
 
 /* 1 if the gated residual and residual entry points (tt_gated_residual_adaln_forward / _backward,
- * tt_adaln_backward_residual) accept (cols, dtype): 3072 columns in any element type, and every
- * other supported row of at most 384 16-byte pieces (3072 two-byte / 1536 four-byte columns).
- * Beyond that those entry points return TT_NORM_EUNSUPPORTED. */
+ * tt_adaln_backward_residual) accept (cols, dtype): every row tt_norm_supported accepts (whole 16-byte pieces,
+ * at most 1024 of them: 8192 two-byte / 4096 four-byte columns).  For other rows those entry points return
+ * TT_NORM_EUNSUPPORTED. */
 int tt_norm_wide_forms_supported(int64_t cols, int dtype);
 
 /* ------------------------------------------------------------------ RMSNorm
@@ -264,8 +266,8 @@ int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void 
  * norm).  The reference runs these as separate elementwise kernels plus the norm; here
  * one pass reads h and attn and writes h2 and out, and one backward pass produces every
  * gradient.  h, attn, h2, out [batch * rows_per_sample, cols]; gate, scale, shift
- * [batch, cols].  Shapes: tt_norm_wide_forms_supported(cols, dtype) -- 3072 columns, or any other
- * supported row of at most 384 16-byte pieces -- else TT_NORM_EUNSUPPORTED.
+ * [batch, cols].  Shapes: tt_norm_wide_forms_supported(cols, dtype) -- every supported row -- else
+ * TT_NORM_EUNSUPPORTED.
  */
 
 int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rstd,

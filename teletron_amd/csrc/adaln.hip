@@ -904,7 +904,7 @@ int tt_gated_residual_adaln_forward(void *h2, void *out, float *mean, float *rst
     if (st != TT_NORM_OK) return st;
     if ((!mean || !rstd) && rows_per_sample > 0)
         return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_forward: null mean/rstd");
-    if (cols != 3072) {
+    if (cols != 3072 || gated_forward_on_wide_rows(cols, dtype)) {
         if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_gated_residual_adaln_forward", cols);
         return anywidth_gated_adaln_forward(h2, out, mean, rstd, h, attn, gate, scale, shift, batch, rows_per_sample, cols,
                                             eps, dtype, (hipStream_t)stream);
@@ -922,6 +922,8 @@ size_t tt_gated_residual_adaln_backward_workspace_bytes(int64_t batch, int64_t r
                                                         int dtype) {
     if (!tt_norm_wide_forms_supported(cols, dtype)) return 0;
     // three sets of column sums (dscale, dshift, dgate) instead of two
+    if (gated_forward_on_wide_rows(cols, dtype))
+        return anywidth_gated_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype);
     return tt_adaln_backward_workspace_bytes(batch, rows_per_sample, cols, dtype) / 2 * 3;
 }
 
@@ -939,7 +941,7 @@ int tt_gated_residual_adaln_backward(void *dh, void *dattn, void *dgate, void *d
     if (dh2 && !aligned16(dh2)) return fail(TT_NORM_EALIGN, "tt_gated_residual_adaln_backward: dh2 not 16-byte aligned");
     if (!dgate || !dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_gated_residual_adaln_backward: null dgate/dscale/dshift/mean/rstd");
-    if (cols != 3072) {
+    if (cols != 3072 || dense_backward_on_wide_rows(cols, dtype) || gated_forward_on_wide_rows(cols, dtype)) {
         if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_gated_residual_adaln_backward", cols);
         return anywidth_gated_adaln_backward(dh, dattn, dgate, dscale, dshift, dout, dh2, h2, attn, gate, scale, mean, rstd,
                                              batch, rows_per_sample, cols, dtype, workspace, workspace_bytes,
@@ -970,7 +972,7 @@ int tt_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void 
     if (st != TT_NORM_OK) return st;
     if (!dscale || !dshift || ((!mean || !rstd) && rows_per_sample > 0))
         return fail(TT_NORM_EINVAL, "tt_adaln_backward_residual: null dscale/dshift/mean/rstd");
-    if (cols != 3072) {
+    if (cols != 3072 || dense_backward_on_wide_rows(cols, dtype)) {
         if (!anywidth_wide_forms_supported(cols, dtype)) return wide_form_unsupported("tt_adaln_backward_residual", cols);
         return anywidth_adaln_backward_residual(dx, dscale, dshift, dout, dres, x, scale, mean, rstd, batch, rows_per_sample,
                                                 cols, dtype, workspace, workspace_bytes, (hipStream_t)stream);

@@ -708,7 +708,7 @@ static size_t backward_scratch(int64_t batch, int64_t rows_per_sample, int64_t c
     RowPlan p;
     if (plan_for(&p, batch, rows_per_sample, geometry_for(cols, dtype), true) != TT_NORM_OK) return 0;
     size_t need = (size_t)p.blocks * nsets * cols * sizeof(float);
-    if (TTN_WIDE_ROWS && nsets <= 2 && widerow_takes(cols, dtype)) {  // dense rows take the other kernels, strided views these
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype)) {  // dense rows take the other kernels, strided views these
         const size_t wide = widerow_backward_workspace_bytes(batch, rows_per_sample, cols, dtype, nsets);
         if (wide == 0) return 0;
         if (wide > need) need = wide;
@@ -760,7 +760,9 @@ static SampleLayout layout_of(int64_t batch, int64_t rows_per_sample, bool seq_f
 }
 
 bool anywidth_wide_forms_supported(int64_t cols, int dtype) {
-    return anywidth_supported(cols, dtype) && geometry_for(cols, dtype).chunks <= 6;
+    if (!anywidth_supported(cols, dtype)) return false;
+    // rows of up to six accesses per lane here; wider dense rows on the wide-row kernels
+    return geometry_for(cols, dtype).chunks <= 6 || (TTN_WIDE_ROWS && widerow_takes(cols, dtype));
 }
 
 template <bool GATED>
@@ -791,6 +793,9 @@ int anywidth_adaln_forward(void *out, float *mean, float *rstd, const void *x, c
 int anywidth_gated_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h, const void *attn,
                                  const void *gate, const void *scale, const void *shift, int64_t batch,
                                  int64_t rows_per_sample, int64_t cols, double eps, int dtype, hipStream_t stream) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_gated_adaln_forward(h2, out, mean, rstd, h, attn, gate, scale, shift, batch, rows_per_sample, cols,
+                                           eps, dtype, stream);
     return adaln_forward_any<true>(out, mean, rstd, h, scale, shift, AdalnExtra{h2, nullptr, attn, gate}, batch,
                                    rows_per_sample, cols, eps, dtype, false, stream);
 }
@@ -839,6 +844,9 @@ int anywidth_adaln_backward_residual(void *dx, void *dscale, void *dshift, const
                                      const void *x, const void *scale, const float *mean, const float *rstd,
                                      int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
                                      size_t ws_bytes, hipStream_t stream) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_adaln_backward_residual(dx, dscale, dshift, g, dres, x, scale, mean, rstd, batch, rows_per_sample,
+                                               cols, dtype, ws, ws_bytes, stream);
     return adaln_backward_any<false, true>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
                                            AdalnExtra{nullptr, dres, nullptr, nullptr}, batch, rows_per_sample, cols, dtype,
                                            ws, ws_bytes, false, stream);
@@ -853,6 +861,9 @@ int anywidth_gated_adaln_backward(void *dh, void *dattn, void *dgate, void *dsca
                                   const void *scale, const float *mean, const float *rstd, int64_t batch,
                                   int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
                                   hipStream_t stream) {
+    if (TTN_WIDE_ROWS && widerow_takes(cols, dtype))
+        return widerow_gated_adaln_backward(dh, dattn, dgate, dscale, dshift, g, dh2, h2, attn, gate, scale, mean, rstd,
+                                            batch, rows_per_sample, cols, dtype, ws, ws_bytes, stream);
     return adaln_backward_any<true, false>(dh, dscale, dshift, dgate, g, h2, scale, mean, rstd,
                                            AdalnExtra{dattn, dh2, attn, gate}, batch, rows_per_sample, cols, dtype, ws,
                                            ws_bytes, false, stream);

@@ -126,6 +126,9 @@ bool widerow_takes(int64_t cols, int dtype);
 // Dense backward calls at a tuned width that run on the wide-row kernels all the same (fp32 rows of 3072 columns: a
 // wavefront that owns such a row has registers for one row buffer only).
 bool dense_backward_on_wide_rows(int64_t cols, int dtype);
+// Measurement builds (-DTTN_GATED_3072_WIDE=1): the gated residual form at 3072 two-byte columns on the wide-row
+// kernels instead of the tuned ones.  False in a shipped build.
+bool gated_forward_on_wide_rows(int64_t cols, int dtype);
 size_t widerow_backward_workspace_bytes(int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, int nsets);
 int widerow_rmsnorm_forward(void *out, float *rstd, const void *x, const void *w, int64_t rows, int64_t cols,
                             double eps, int dtype, hipStream_t stream);
@@ -137,5 +140,17 @@ int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, co
 int widerow_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x, const void *scale,
                            const float *mean, const float *rstd, int64_t batch, int64_t rows_per_sample, int64_t cols,
                            int dtype, void *ws, size_t ws_bytes, bool seq_first, hipStream_t stream);
+int widerow_gated_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h, const void *attn,
+                                const void *gate, const void *scale, const void *shift, int64_t batch,
+                                int64_t rows_per_sample, int64_t cols, double eps, int dtype, hipStream_t stream);
+int widerow_gated_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift, const void *g,
+                                 const void *dh2, const void *h2, const void *attn, const void *gate,
+                                 const void *scale, const float *mean, const float *rstd, int64_t batch,
+                                 int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                                 hipStream_t stream);
+int widerow_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *g, const void *dres,
+                                    const void *x, const void *scale, const float *mean, const float *rstd,
+                                    int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                                    size_t ws_bytes, hipStream_t stream);
 
 }  // namespace ttn

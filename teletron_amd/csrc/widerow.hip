@@ -54,7 +54,11 @@
 
 namespace ttn {
 
-constexpr int kWidePiecesMin = 385;  // narrower rows belong to the one-wavefront-per-row kernels
+#ifndef TTN_GATED_3072_WIDE
+#define TTN_GATED_3072_WIDE 0
+#endif
+// narrower rows belong to the one-wavefront-per-row kernels
+constexpr int kWidePiecesMin = TTN_GATED_3072_WIDE ? 384 : 385;
 
 // Which of this lane's CH accesses lie inside a row of `pieces` 16-byte pieces, for wavefront `wave`.
 template <int CH>
@@ -357,11 +361,15 @@ __global__ __launch_bounds__(kRowThreads) void wide_rmsnorm_bwd_kernel(T *__rest
 
 // -------------------------------------------------------------------- AdaLN
 
-template <typename T, int CH>
+// GATED: the row that is normalised is h2 = rnd(x + rnd(attn * gate[b])), which is written out too (the gated
+// residual update in front of the norm; same form as the kernels of adaln.hip / anywidth.hip).
+template <typename T, int CH, bool GATED>
 __global__ __launch_bounds__(kRowThreads) void wide_adaln_fwd_kernel(T *__restrict__ out, float *__restrict__ mean,
                                                                      float *__restrict__ rstd, const T *__restrict__ x,
                                                                      const T *__restrict__ scale,
-                                                                     const T *__restrict__ shift, int64_t rows_per_sample,
+                                                                     const T *__restrict__ shift, T *__restrict__ h2_out,
+                                                                     const T *__restrict__ attn, const T *__restrict__ gate,
+                                                                     int64_t rows_per_sample,
                                                                      const SampleLayout lay, int blocks_per_sample, int C,
                                                                      int ppw, float eps) {
     using E = Elem<T>;
@@ -405,19 +413,52 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_fwd_kernel(T *__restri
         }
     }
 
+    [[maybe_unused]] u32x4 qr[GATED ? CH : 1];  // gate[b], packed
+    if constexpr (GATED) {
+#pragma unroll
+        for (int k = 0; k < CH; ++k)
+            qr[k] = m.in[k] ? load16(reinterpret_cast<const u32x4 *>(gate + b * C + slice) + k * kWaveSize + lane)
+                            : u32x4{0, 0, 0, 0};
+    }
+
     int parity = 0;
     u32x4 xr[CH];
-    if (slot < rows_per_sample)
+    [[maybe_unused]] u32x4 ar[GATED ? CH : 1];
+    if (slot < rows_per_sample) {
         wide_load<CH>(xr, reinterpret_cast<const u32x4 *>(x + lay.row(b, slot) * C + slice) + lane, true, m);
+        if constexpr (GATED)
+            wide_load<CH>(ar, reinterpret_cast<const u32x4 *>(attn + lay.row(b, slot) * C + slice) + lane, true, m);
+    }
     for (int64_t rs = slot; rs < rows_per_sample; rs += blocks_per_sample, parity ^= 1) {
         if constexpr (!kParamsF32) {
             keep_packed(tr);
             keep_packed(hr);
         }
+        if constexpr (GATED) keep_packed(qr);
         const int64_t row = lay.row(b, rs);
 #if !TTN_WIDE_FWD_PREFETCH
-        if (rs != slot) wide_load<CH>(xr, reinterpret_cast<const u32x4 *>(x + row * C + slice) + lane, true, m);
+        if (rs != slot) {
+            wide_load<CH>(xr, reinterpret_cast<const u32x4 *>(x + row * C + slice) + lane, true, m);
+            if constexpr (GATED) wide_load<CH>(ar, reinterpret_cast<const u32x4 *>(attn + row * C + slice) + lane, true, m);
+        }
 #endif
+        if constexpr (GATED) {
+            const RowWriter<0> wh(h2_out + row * C + slice, lane * 16);
+#pragma unroll
+            for (int k = 0; k < CH; ++k) {
+                float hv[VEC], av[VEC], gv[VEC];
+                E::unpack(xr[k], hv);
+                E::unpack(ar[k], av);
+                E::unpack(qr[k], gv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) av[j] *= gv[j];
+                E::round(av);  // attn * gate materialised in the element type
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) hv[j] += av[j];
+                xr[k] = E::pack(hv);  // h2: the new residual stream, and the row that is normalised
+                if (m.in[k]) wh.put(k * kWaveSize, xr[k]);
+            }
+        }
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < CH; ++k) {
@@ -453,6 +494,9 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_fwd_kernel(T *__restri
         const int64_t rs_next = rs + blocks_per_sample;
         const bool more = rs_next < rows_per_sample;
         wide_load<CH>(xn, reinterpret_cast<const u32x4 *>(x + lay.row(b, more ? rs_next : rs) * C + slice) + lane, more, m);
+        [[maybe_unused]] u32x4 an[GATED ? CH : 1];
+        if constexpr (GATED)
+            wide_load<CH>(an, reinterpret_cast<const u32x4 *>(attn + lay.row(b, more ? rs_next : rs) * C + slice) + lane, more, m);
 #endif
         const float *sl = xch[parity];
         const float mu = wide_total<2>(sl, 0) / (float)C;
@@ -497,18 +541,29 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_fwd_kernel(T *__restri
 #if TTN_WIDE_FWD_PREFETCH
 #pragma unroll
         for (int k = 0; k < CH; ++k) xr[k] = xn[k];
+        if constexpr (GATED) {
+#pragma unroll
+            for (int k = 0; k < CH; ++k) ar[k] = an[k];
+        }
 #endif
     }
 }
 
-template <typename T, int CH>
+// GATED: x is the saved h2; dx = dh = rnd(rnd(dx of the norm) + e) with e the gradient arriving at h2 from its other
+// use (may be null), da = rnd(dh * gate[b]) is written too and dgate[b] += rnd(dh * attn) is a third set of column
+// sums.  RES: dx = rnd(rnd(dx of the norm) + e), e the gradient the input receives from its other consumer.
+template <typename T, int CH, bool GATED, bool RES>
 __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restrict__ dx, float *__restrict__ partial,
                                                                      const T *__restrict__ g, const T *__restrict__ x,
                                                                      const T *__restrict__ scale,
                                                                      const float *__restrict__ mean,
-                                                                     const float *__restrict__ rstd, int64_t rows_per_sample,
+                                                                     const float *__restrict__ rstd, T *__restrict__ da,
+                                                                     const T *__restrict__ e, const T *__restrict__ attn,
+                                                                     const T *__restrict__ gate, int64_t rows_per_sample,
                                                                      const SampleLayout lay, int blocks_per_sample, int C,
                                                                      int ppw) {
+    static_assert(!(GATED && RES), "the gated form handles e itself");
+    constexpr int NSETS = GATED ? 3 : 2;
     using E = Elem<T>;
     constexpr int VEC = E::VEC;
     __shared__ float xch[2][kRowWaves * 2];
@@ -531,9 +586,16 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
         for (int j = 0; j < VEC; ++j) v[j] = 1.0f + v[j];
         tp.set(k, E::pack(v));
     }
-    float acc[2][CH][VEC];  // [0] = dscale, [1] = dshift
+    [[maybe_unused]] u32x4 qr[GATED ? CH : 1];  // gate[sample], packed
+    if constexpr (GATED) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+        for (int k = 0; k < CH; ++k)
+            qr[k] = m.in[k] ? load16(reinterpret_cast<const u32x4 *>(gate + smp * C + slice) + k * kWaveSize + lane)
+                            : u32x4{0, 0, 0, 0};
+    }
+    float acc[NSETS][CH][VEC];  // [0] = dscale, [1] = dshift, [2] = dgate
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s)
 #pragma unroll
         for (int k = 0; k < CH; ++k)
 #pragma unroll
@@ -541,6 +603,7 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
 
     struct Row {
         u32x4 g[CH], x[CH];
+        u32x4 e[(GATED || RES) ? CH : 1], a[GATED ? CH : 1];
         float r, mu;
         int64_t row;
     };
@@ -549,6 +612,9 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
         b.row = lay.row(smp, ok ? rs : 0);
         wide_load<CH>(b.g, reinterpret_cast<const u32x4 *>(g + b.row * C + slice) + lane, ok, m);
         wide_load<CH>(b.x, reinterpret_cast<const u32x4 *>(x + b.row * C + slice) + lane, ok, m);
+        if constexpr (GATED || RES)
+            wide_load<CH>(b.e, reinterpret_cast<const u32x4 *>(e + b.row * C + slice) + lane, ok && e != nullptr, m);
+        if constexpr (GATED) wide_load<CH>(b.a, reinterpret_cast<const u32x4 *>(attn + b.row * C + slice) + lane, ok, m);
         const int64_t srow = wave_uniform(b.row);
         b.r = ok ? rstd[srow] : 0.0f;
         b.mu = ok ? mean[srow] : 0.0f;
@@ -593,7 +659,9 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
         const float K1 = k1 * r;
         const float K0 = fmaf(k1, nmr, k0);
 
-        const RowWriter<TTN_WIDE_BWD_STORE> wd(dx + b.row * C + slice, lane * 16);
+        const RowWriter<GATED ? 0 : TTN_WIDE_BWD_STORE> wd(dx + b.row * C + slice, lane * 16);
+        const RowWriter<0> wa(GATED ? da + b.row * C + slice : nullptr, lane * 16);
+        if constexpr (GATED) keep_packed(qr);
 #pragma unroll
         for (int k = 0; k < CH; ++k) {
             float gx[VEC], xv[VEC], o[VEC], xn[VEC];
@@ -604,7 +672,30 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
                 o[j] = fmaf(r, gx[j], fmaf(xv[j], K1, K0));
                 xn[j] = centred<T>(xv[j], mu, r, nmr);
             }
-            if (m.in[k]) wd.put(k * kWaveSize, E::pack(o));
+            if constexpr (GATED || RES) {
+                float ev[VEC];
+                E::round(o);  // the norm's dx, materialised in the element type
+                E::unpack(b.e[k], ev);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o[j] += ev[j];
+            }
+            const u32x4 dxp = E::pack(o);
+            if (m.in[k]) wd.put(k * kWaveSize, dxp);
+            if constexpr (GATED) {
+                float av[VEC], qv[VEC];
+                E::unpack(dxp, o);  // dh as stored
+                E::unpack(b.a[k], av);
+                E::unpack(qr[k], qv);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    qv[j] *= o[j];
+                    av[j] *= o[j];
+                }
+                if (m.in[k]) wa.put(k * kWaveSize, E::pack(qv));
+                E::round(av);  // dh*attn materialised in the element type before the column sum
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[2][k][j] += av[j];
+            }
             add_elements<T>(acc[1][k], b.g[k], one_lo, one_hi);                // dshift += g (padding: g = 0)
             add_rounded_products<T>(acc[0][k], b.g[k], xn, one_lo, one_hi);    // dscale += rnd(g * rnd(xhat))
         }
@@ -632,7 +723,7 @@ __global__ __launch_bounds__(kRowThreads) void wide_adaln_bwd_kernel(T *__restri
         }
 #endif
     }
-    wide_store_partials<T, CH, 2>(acc, partial + (int64_t)blockIdx.x * (2 * C), C, slice, lane, m);
+    wide_store_partials<T, CH, NSETS>(acc, partial + (int64_t)blockIdx.x * (NSETS * C), C, slice, lane, m);
 }
 
 // ------------------------------------------------------------------ host side
@@ -645,6 +736,9 @@ bool widerow_takes(int64_t cols, int dtype) {
 #ifndef TTN_F32_3072_BWD_WIDE
 #define TTN_F32_3072_BWD_WIDE 1
 #endif
+bool gated_forward_on_wide_rows(int64_t cols, int dtype) {
+    return TTN_GATED_3072_WIDE && TTN_WIDE_ROWS && dtype != TT_NORM_F32 && cols == 3072;
+}
 bool dense_backward_on_wide_rows(int64_t cols, int dtype) {
     return TTN_F32_3072_BWD_WIDE && TTN_WIDE_ROWS && dtype == TT_NORM_F32 && cols == 3072;
 }
@@ -752,9 +846,17 @@ int widerow_rmsnorm_backward(void *dx, void *dw, const void *g, const void *x, c
     return launch_colreduce(dw, nullptr, nullptr, (const float *)ws, 1, p.blocks_per_sample, cols, cols, dtype, stream);
 }
 
-int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale, const void *shift,
-                          int64_t batch, int64_t rows_per_sample, int64_t cols, double eps, int dtype, bool seq_first,
-                          hipStream_t stream) {
+struct WideExtra {  // operands of the gated / residual forms (null otherwise)
+    void *h2_or_da;    // forward: h2 out; backward: da out
+    const void *e;     // backward: the gradient arriving at h2 / at the input from its other use
+    const void *attn;
+    const void *gate;
+};
+
+template <bool GATED>
+static int wide_adaln_forward_t(void *out, float *mean, float *rstd, const void *x, const void *scale,
+                                const void *shift, const WideExtra &ex, int64_t batch, int64_t rows_per_sample,
+                                int64_t cols, double eps, int dtype, bool seq_first, hipStream_t stream) {
     if (rows_per_sample == 0) return TT_NORM_OK;
     RowPlan p;
     int st = TT_NORM_OK;
@@ -764,12 +866,14 @@ int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, co
         RowKernelProfile prof(stream);
 #define CALL(T, CH)                                                                                         \
     do {                                                                                                    \
-        static const int per_cu = resident_blocks_per_cu(wide_adaln_fwd_kernel<T, CH>, TTN_WIDE_FWD_BLOCKS_PER_CU); \
+        static const int per_cu =                                                                           \
+            resident_blocks_per_cu(wide_adaln_fwd_kernel<T, CH, GATED>, TTN_WIDE_FWD_BLOCKS_PER_CU);        \
         st = wide_plan(&p, batch, rows_per_sample, per_cu, TTN_WIDE_ADALN_FWD_ROWS_PER_BLOCK);              \
         if (st != TT_NORM_OK) return st;                                                                    \
-        wide_adaln_fwd_kernel<T, CH><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(           \
-            (T *)out, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift, rows_per_sample, lay,   \
-            p.blocks_per_sample, (int)cols, ppw, (float)eps);                                               \
+        wide_adaln_fwd_kernel<T, CH, GATED><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(    \
+            (T *)out, mean, rstd, (const T *)x, (const T *)scale, (const T *)shift, (T *)ex.h2_or_da,       \
+            (const T *)ex.attn, (const T *)ex.gate, rows_per_sample, lay, p.blocks_per_sample, (int)cols,   \
+            ppw, (float)eps);                                                                               \
     } while (0)
         TTN_WIDE_DISPATCH(dtype, ch, CALL);
 #undef CALL
@@ -777,33 +881,85 @@ int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, co
     return check_launch("adaln forward launch (wide rows)");
 }
 
-int widerow_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x, const void *scale,
-                           const float *mean, const float *rstd, int64_t batch, int64_t rows_per_sample, int64_t cols,
-                           int dtype, void *ws, size_t ws_bytes, bool seq_first, hipStream_t stream) {
+int widerow_adaln_forward(void *out, float *mean, float *rstd, const void *x, const void *scale, const void *shift,
+                          int64_t batch, int64_t rows_per_sample, int64_t cols, double eps, int dtype, bool seq_first,
+                          hipStream_t stream) {
+    return wide_adaln_forward_t<false>(out, mean, rstd, x, scale, shift, WideExtra{nullptr, nullptr, nullptr, nullptr},
+                                       batch, rows_per_sample, cols, eps, dtype, seq_first, stream);
+}
+
+int widerow_gated_adaln_forward(void *h2, void *out, float *mean, float *rstd, const void *h, const void *attn,
+                                const void *gate, const void *scale, const void *shift, int64_t batch,
+                                int64_t rows_per_sample, int64_t cols, double eps, int dtype, hipStream_t stream) {
+    return wide_adaln_forward_t<true>(out, mean, rstd, h, scale, shift, WideExtra{h2, nullptr, attn, gate}, batch,
+                                      rows_per_sample, cols, eps, dtype, false, stream);
+}
+
+template <bool GATED, bool RES>
+static int wide_adaln_backward_t(void *dx, void *dscale, void *dshift, void *dgate, const void *g, const void *x,
+                                 const void *scale, const float *mean, const float *rstd, const WideExtra &ex,
+                                 int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                                 size_t ws_bytes, bool seq_first, hipStream_t stream) {
+    constexpr int NSETS = GATED ? 3 : 2;
     if (rows_per_sample == 0)
-        return launch_colreduce(dscale, dshift, nullptr, nullptr, batch, 0, cols, 2 * cols, dtype, stream);
+        return launch_colreduce(dscale, dshift, dgate, nullptr, batch, 0, cols, NSETS * cols, dtype, stream);
     RowPlan p;
-    int st = wide_plan(&p, batch, rows_per_sample, TTN_WIDE_BWD_BLOCKS_PER_CU);
-    if (st != TT_NORM_OK) return st;
-    const size_t need = (size_t)p.blocks * 2 * cols * sizeof(float);
-    if (!ws || ws_bytes < need)
-        return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
-    if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "adaln backward: workspace %p not 16-byte aligned", ws);
+    int st = TT_NORM_OK;
     const SampleLayout lay = seq_first ? SampleLayout{1, batch} : SampleLayout{rows_per_sample, 1};
     const int ch = wide_chunks(cols, dtype), ppw = wide_pieces_per_wave(cols, dtype);
     {
         RowKernelProfile prof(stream);
+        // The same grid for the plain, gated and residual forms of a shape, so that their column sums are added in
+        // the same order and the fused forms stay bit-identical to their parts; an instantiation whose registers
+        // leave room for one workgroup per compute unit only (gated, four accesses per lane) runs its grid in two
+        // rounds.
 #define CALL(T, CH)                                                                                         \
-    wide_adaln_bwd_kernel<T, CH><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>(               \
-        (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)scale, mean, rstd, rows_per_sample, lay, \
-        p.blocks_per_sample, (int)cols, ppw)
+    do {                                                                                                    \
+        st = wide_plan(&p, batch, rows_per_sample, TTN_WIDE_BWD_BLOCKS_PER_CU);                             \
+        if (st != TT_NORM_OK) return st;                                                                    \
+        const size_t need = (size_t)p.blocks * NSETS * cols * sizeof(float);                                \
+        if (!ws || ws_bytes < need)                                                                         \
+            return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need); \
+        if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "adaln backward: workspace %p not 16-byte aligned", ws); \
+        wide_adaln_bwd_kernel<T, CH, GATED, RES><<<dim3((unsigned)p.blocks), dim3(kRowThreads), 0, stream>>>( \
+            (T *)dx, (float *)ws, (const T *)g, (const T *)x, (const T *)scale, mean, rstd, (T *)ex.h2_or_da, \
+            (const T *)ex.e, (const T *)ex.attn, (const T *)ex.gate, rows_per_sample, lay, p.blocks_per_sample, \
+            (int)cols, ppw);                                                                                \
+    } while (0)
         TTN_WIDE_DISPATCH(dtype, ch, CALL);
 #undef CALL
     }
     st = check_launch("adaln backward launch (wide rows)");
     if (st != TT_NORM_OK) return st;
-    return launch_colreduce(dscale, dshift, nullptr, (const float *)ws, batch, p.blocks_per_sample, cols, 2 * cols, dtype,
-                            stream);
+    return launch_colreduce(dscale, dshift, dgate, (const float *)ws, batch, p.blocks_per_sample, cols, NSETS * cols,
+                            dtype, stream);
+}
+
+int widerow_adaln_backward(void *dx, void *dscale, void *dshift, const void *g, const void *x, const void *scale,
+                           const float *mean, const float *rstd, int64_t batch, int64_t rows_per_sample, int64_t cols,
+                           int dtype, void *ws, size_t ws_bytes, bool seq_first, hipStream_t stream) {
+    return wide_adaln_backward_t<false, false>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
+                                               WideExtra{nullptr, nullptr, nullptr, nullptr}, batch, rows_per_sample,
+                                               cols, dtype, ws, ws_bytes, seq_first, stream);
+}
+
+int widerow_adaln_backward_residual(void *dx, void *dscale, void *dshift, const void *g, const void *dres,
+                                    const void *x, const void *scale, const float *mean, const float *rstd,
+                                    int64_t batch, int64_t rows_per_sample, int64_t cols, int dtype, void *ws,
+                                    size_t ws_bytes, hipStream_t stream) {
+    return wide_adaln_backward_t<false, true>(dx, dscale, dshift, nullptr, g, x, scale, mean, rstd,
+                                              WideExtra{nullptr, dres, nullptr, nullptr}, batch, rows_per_sample, cols,
+                                              dtype, ws, ws_bytes, false, stream);
+}
+
+int widerow_gated_adaln_backward(void *dh, void *dattn, void *dgate, void *dscale, void *dshift, const void *g,
+                                 const void *dh2, const void *h2, const void *attn, const void *gate,
+                                 const void *scale, const float *mean, const float *rstd, int64_t batch,
+                                 int64_t rows_per_sample, int64_t cols, int dtype, void *ws, size_t ws_bytes,
+                                 hipStream_t stream) {
+    return wide_adaln_backward_t<true, false>(dh, dscale, dshift, dgate, g, h2, scale, mean, rstd,
+                                              WideExtra{dattn, dh2, attn, gate}, batch, rows_per_sample, cols, dtype, ws,
+                                              ws_bytes, false, stream);
 }
 
 }  // namespace ttn

@@ -50,7 +50,6 @@ except ImportError as exc:  # pragma: no cover - exercised only on an unbuilt tr
                 "build them with `python -m teletron_amd.build`.", exc)
 
 TUNED_COLS = (128, 3072)  # the reference's two shapes (the tuned kernels)
-_WIDE_FORM_PIECES = 384   # gated / residual forms: 3072 columns, or any row of up to this many 16-byte pieces
 _ELEM_BYTES = {torch.bfloat16: 2, torch.float16: 2, torch.float32: 4}
 _MAX_PIECES = 1024  # 16-byte pieces per row the kernels are built for
 
@@ -67,7 +66,7 @@ def cols_supported(cols: int, dtype: torch.dtype) -> bool:
 
 def wide_forms_supported(cols: int, dtype: torch.dtype) -> bool:
     """Whether the gated residual + AdaLN and the stream-keeping AdaLN take rows of `cols` elements."""
-    return cols_supported(cols, dtype) and (cols == 3072 or cols * _ELEM_BYTES[dtype] // 16 <= _WIDE_FORM_PIECES)
+    return cols_supported(cols, dtype)   # every supported row: tuned, any-width and wide-row kernels all have the forms
 
 
 def _unsupported(cols: int, dtype: torch.dtype) -> str:
@@ -189,8 +188,7 @@ class AdaLNResidualFunction(Function):
     itself, handed back as an output for the caller to continue the residual stream with
     (dit_layerspec.py:126-131 then :152).  Routing the stream through the Function lets backward add the
     gradient it collected downstream to the norm's dx inside the kernel, in place of the separate
-    accumulation pass autograd runs when a tensor has two consumers.  3072 columns, or any supported row of up
-    to 3072 two-byte / 1536 four-byte columns."""
+    accumulation pass autograd runs when a tensor has two consumers.  Any supported row."""
 
     @staticmethod
     def forward(ctx, x, scale, shift, epsilon):
@@ -198,8 +196,7 @@ class AdaLNResidualFunction(Function):
         _require_gpu(x, "AdaLNResidualFunction")
         cols = x.shape[-1]
         if x.dtype not in _ELEM_BYTES or not wide_forms_supported(cols, x.dtype):
-            raise ValueError(f"AdaLNResidualFunction: {_unsupported(cols, x.dtype)}; rows of at most 3072 two-byte / "
-                             "1536 four-byte columns, or 3072 columns")
+            raise ValueError(f"AdaLNResidualFunction: {_unsupported(cols, x.dtype)}")
         x_c = _aligned_contiguous(x)
         scale_c, shift_c = scale.contiguous().to(x.dtype), shift.contiguous().to(x.dtype)
         if scale_c.numel() % cols or shift_c.numel() != scale_c.numel():
@@ -288,8 +285,7 @@ class GatedResidualAdaLNFunction(Function):
         _require_gpu(h, "GatedResidualAdaLNFunction")
         cols = h.shape[-1]
         if h.dtype not in _ELEM_BYTES or not wide_forms_supported(cols, h.dtype):
-            raise ValueError(f"GatedResidualAdaLNFunction: {_unsupported(cols, h.dtype)}; rows of at most 3072 two-byte "
-                             "/ 1536 four-byte columns, or 3072 columns")
+            raise ValueError(f"GatedResidualAdaLNFunction: {_unsupported(cols, h.dtype)}")
         if attn.shape != h.shape:
             raise ValueError(f"attn {tuple(attn.shape)} must have the shape of h {tuple(h.shape)}")
         mods = [t.contiguous().to(h.dtype) for t in (gate, scale, shift)]

@@ -64,7 +64,8 @@ static void predicates() {
             EXPECT(!t || s);   // tuned shapes are supported shapes
             EXPECT(!w || s);   // the wide forms exist for supported shapes only
         }
-    EXPECT(tt_norm_wide_forms_supported(3072, TT_NORM_F32) == 1 && tt_norm_wide_forms_supported(1540, TT_NORM_F32) == 0);
+    EXPECT(tt_norm_wide_forms_supported(3072, TT_NORM_F32) == 1 && tt_norm_wide_forms_supported(1540, TT_NORM_F32) == 1);
+    EXPECT(tt_norm_wide_forms_supported(4100, TT_NORM_F32) == 0 && tt_norm_wide_forms_supported(3076, TT_NORM_BF16) == 0);
 }
 
 static void row_plans() {
@@ -126,12 +127,12 @@ static void argument_checks(bool have_gpu) {
            TT_NORM_EINVAL);
     EXPECT(tt_rmsnorm_rope_forward_strided(a, f, b, c, f, f, 2, 1, 2, 3, 0, 0, 64, 64, 1e-6, TT_NORM_BF16, nullptr) ==
            TT_NORM_EUNSUPPORTED);
-    // gated / residual forms beyond 384 pieces
-    EXPECT(tt_gated_residual_adaln_forward(a, b, f, f, a, b, c, d, a, 1, 4, 3080, 1e-6, TT_NORM_BF16, nullptr) ==
+    // gated / residual forms on rows that are not whole 16-byte pieces, or wider than 1024 of them
+    EXPECT(tt_gated_residual_adaln_forward(a, b, f, f, a, b, c, d, a, 1, 4, 3076, 1e-6, TT_NORM_BF16, nullptr) ==
            TT_NORM_EUNSUPPORTED);
-    EXPECT(tt_adaln_backward_residual(a, b, c, d, a, b, c, f, f, 1, 4, 1540, TT_NORM_F32, nullptr, 0, nullptr) ==
+    EXPECT(tt_adaln_backward_residual(a, b, c, d, a, b, c, f, f, 1, 4, 4100, TT_NORM_F32, nullptr, 0, nullptr) ==
            TT_NORM_EUNSUPPORTED);
-    EXPECT(tt_gated_residual_adaln_backward_workspace_bytes(1, 4, 4096, TT_NORM_BF16) == 0);
+    EXPECT(tt_gated_residual_adaln_backward_workspace_bytes(1, 4, 8200, TT_NORM_BF16) == 0);
     // the entry point with static scratch: a shape that cannot fit is refused before anything else happens
     EXPECT(tt_adaln_backward_static(a, b, c, d, a, b, f, f, -1, 4, 3072, TT_NORM_BF16, nullptr) == TT_NORM_EINVAL);
     // the event hook: both or neither

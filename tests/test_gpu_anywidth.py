@@ -280,7 +280,10 @@ def test_strided_qk_norm_at_other_head_dims(capi, gpu_device, D, dtype, B, S, H)
 
 
 @pytest.mark.parametrize("C,dtype,B,S,with_h2", [(1536, BF, 2, 515, True), (1024, HF, 3, 130, False), (512, F32, 2, 77, True),
-                                                 (2048, BF, 1, 300, True), (64, BF, 2, 1001, True), (1536, F32, 1, 65, False)])
+                                                 (2048, BF, 1, 300, True), (64, BF, 2, 1001, True), (1536, F32, 1, 65, False),
+                                                 # rows of more than 384 pieces: four wavefronts per row
+                                                 (4096, BF, 2, 515, True), (5120, HF, 1, 130, False), (8192, BF, 3, 67, True),
+                                                 (3080, BF, 1, 1100, True), (2048, F32, 2, 77, True), (4096, F32, 1, 33, False)])
 def test_gated_residual_adaln_at_other_widths(capi, gpu_device, C, dtype, B, S, with_h2):
     h, a, q, sc, sh, go, g2 = O.make_gated_inputs(B, S, C, dtype, seed=C + S, with_grad_h2=with_h2)
     want = O.eager_gated_residual_adaln_fwd_bwd(h, a, q, sc, sh, go, g2)
@@ -312,7 +315,8 @@ def test_gated_residual_adaln_at_other_widths(capi, gpu_device, C, dtype, B, S, 
         colsum_ok(dsh, want[6], go.float(), 1, "dshift")
 
 
-@pytest.mark.parametrize("C,dtype", [(1536, BF), (1024, HF), (768, F32), (128, BF)])
+@pytest.mark.parametrize("C,dtype", [(1536, BF), (1024, HF), (768, F32), (128, BF), (4096, BF), (6152, HF), (1540, F32),
+                                     (8192, BF)])
 def test_adaln_backward_residual_at_other_widths(capi, gpu_device, C, dtype):
     d = O.make_adaln_inputs(2, 301, C, dtype, seed=C)
     other = O.make_adaln_inputs(2, 301, C, dtype, seed=C + 1)["grad"]
@@ -364,9 +368,9 @@ def test_functions_take_the_wide_forms_at_other_widths(gpu_device):
     torch.autograd.backward([out2, same * 1.0], [go.to(gpu_device), g2.to(gpu_device)])
     assert x.grad is not None and x.grad.shape == h.shape
     with pytest.raises(ValueError, match="unsupported cols|rows of at most"):
-        FL.gated_residual_layer_norm(torch.zeros(1, 4, 4096, dtype=BF, device=gpu_device),
-                                     torch.zeros(1, 4, 4096, dtype=BF, device=gpu_device),
-                                     *(torch.zeros(1, 4096, dtype=BF, device=gpu_device) for _ in range(3)), eps=EPS)
+        FL.gated_residual_layer_norm(torch.zeros(1, 4, 4100, dtype=BF, device=gpu_device),
+                                     torch.zeros(1, 4, 4100, dtype=BF, device=gpu_device),
+                                     *(torch.zeros(1, 4100, dtype=BF, device=gpu_device) for _ in range(3)), eps=EPS)
     B, S, H, D = 1, 101, 4, 64
     gen = torch.Generator().manual_seed(64)
     mixed = torch.randn(B, S, H, 3 * D, generator=gen).bfloat16()

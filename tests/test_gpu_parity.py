@@ -366,8 +366,11 @@ def test_full_size_gated_residual_adaln_properties(capi, gpu_device):
 
 def test_gated_residual_adaln_rejects_other_widths(capi, gpu_device):
     mk = lambda *shape: torch.zeros(*shape, device=gpu_device, dtype=torch.bfloat16)
-    with pytest.raises(capi.NormError) as e:     # rows of more than six 16-byte accesses per lane (other than 3072)
-        capi.gated_residual_adaln_forward(mk(1, 8, 4096), mk(1, 8, 4096), mk(1, 4096), mk(1, 4096), mk(1, 4096), EPS)
+    with pytest.raises(capi.NormError) as e:     # rows that are not whole 16-byte pieces, or too wide
+        capi.gated_residual_adaln_forward(mk(1, 8, 4100), mk(1, 8, 4100), mk(1, 4100), mk(1, 4100), mk(1, 4100), EPS)
+    assert e.value.status == 2
+    with pytest.raises(capi.NormError) as e:
+        capi.gated_residual_adaln_forward(mk(1, 8, 8200), mk(1, 8, 8200), mk(1, 8200), mk(1, 8200), mk(1, 8200), EPS)
     assert e.value.status == 2
     # zero rows: a no-op forward and all-zero parameter gradients
     h2, out, mean, rstd = capi.gated_residual_adaln_forward(mk(2, 0, 3072), mk(2, 0, 3072), mk(2, 3072),

@@ -96,7 +96,7 @@ def _wide_cases(seed, n):
     for _ in range(n):
         dtype = rng.choice([BF, BF, HF, F32])
         piece = 4 if dtype == F32 else 8
-        pieces = rng.choice([rng.randint(1, 16), rng.randint(1, 64), rng.randint(1, 384), 384])
+        pieces = rng.choice([rng.randint(1, 16), rng.randint(1, 64), rng.randint(1, 384), 384, rng.randint(385, 1024)])
         out.append((pieces * piece, dtype, rng.randint(1, 4), rng.randint(1, 400), rng.random() < 0.7))
     return out
 

@@ -27,7 +27,7 @@ def test_c_abi_exports_every_declared_symbol():
     for n in names:
         assert hasattr(L, n), f"{n} declared in teletron_norm.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert L.tt_norm_abi_version() == 2
+    assert L.tt_norm_abi_version() == 3
     assert L.tt_norm_status_string(0) == b"ok"
     assert L.tt_norm_status_string(4).startswith(b"workspace")
     assert L.tt_norm_supported(3072, capi.BF16) == 1 and L.tt_norm_supported(128, capi.F32) == 1
@@ -84,7 +84,7 @@ def test_probe_library_is_separate_and_exports_its_header():
 
 
 def test_wide_forms_query_matches_the_python_gate():
-    """tt_norm_wide_forms_supported: 3072 columns, or any supported row of up to 384 16-byte pieces; the
+    """tt_norm_wide_forms_supported: every supported row (whole 16-byte pieces, at most 1024 of them); the
     Python-side gate of the gated / residual Functions says the same for every width."""
     from teletron_amd import capi
     from teletron_amd import fusedlayers as FL
@@ -92,14 +92,15 @@ def test_wide_forms_query_matches_the_python_gate():
     for dt, code in ((torch.bfloat16, capi.BF16), (torch.float16, capi.F16), (torch.float32, capi.F32)):
         for cols in list(range(0, 8200, 4)) + [3072, 3080, 1536, 1540, 8192]:
             assert bool(L.tt_norm_wide_forms_supported(cols, code)) == FL.wide_forms_supported(cols, dt), (cols, dt)
-    assert L.tt_norm_wide_forms_supported(3072, capi.F32) == 1 and L.tt_norm_wide_forms_supported(1540, capi.F32) == 0
-    assert L.tt_norm_wide_forms_supported(3080, capi.BF16) == 0 and L.tt_norm_wide_forms_supported(3064, capi.BF16) == 1
+    assert L.tt_norm_wide_forms_supported(3072, capi.F32) == 1 and L.tt_norm_wide_forms_supported(1540, capi.F32) == 1
+    assert L.tt_norm_wide_forms_supported(3080, capi.BF16) == 1 and L.tt_norm_wide_forms_supported(8192, capi.BF16) == 1
+    assert L.tt_norm_wide_forms_supported(4100, capi.F32) == 0 and L.tt_norm_wide_forms_supported(3076, capi.BF16) == 0
     assert L.tt_norm_wide_forms_supported(3072, 7) == 0
-    # beyond it the three entry points answer TT_NORM_EUNSUPPORTED before touching a pointer
-    assert L.tt_gated_residual_adaln_forward(*([None] * 9), 1, 4, 3080, 1e-6, capi.BF16, None) == 2
-    assert L.tt_gated_residual_adaln_backward(*([None] * 13), 1, 4, 4096, capi.BF16, None, 0, None) == 2
-    assert L.tt_adaln_backward_residual(*([None] * 9), 1, 4, 1540, capi.F32, None, 0, None) == 2
-    assert L.tt_gated_residual_adaln_backward_workspace_bytes(1, 4, 3080, capi.BF16) == 0
+    # other rows: the three entry points answer TT_NORM_EUNSUPPORTED before touching a pointer
+    assert L.tt_gated_residual_adaln_forward(*([None] * 9), 1, 4, 3076, 1e-6, capi.BF16, None) == 2
+    assert L.tt_gated_residual_adaln_backward(*([None] * 13), 1, 4, 8200, capi.BF16, None, 0, None) == 2
+    assert L.tt_adaln_backward_residual(*([None] * 9), 1, 4, 4100, capi.F32, None, 0, None) == 2
+    assert L.tt_gated_residual_adaln_backward_workspace_bytes(1, 4, 3076, capi.BF16) == 0
 
 
 def test_extension_modules_expose_reference_names():
