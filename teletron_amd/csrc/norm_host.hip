@@ -135,9 +135,84 @@ __global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_kernel(
     wave_clock_mark(kClockColReduce, 1);
 }
 
+// The same sums, 128 columns per workgroup: thread (tx, ty) of 32 x 32 owns the four adjacent columns of one
+// 16-byte piece and adds partial rows ty, ty+32, ... in ascending order with up to eight loads in flight; then
+// one thread per column adds the 32 strands in ascending ty.  Same association order as colreduce_kernel (so
+// the same bits), a quarter of the workgroups, 16-byte loads.  ncols must be a multiple of four and the partial
+// rows 16-byte aligned.
+constexpr int kRedWideCols = 4 * kRedCols;
+
+template <typename T>
+__global__ __launch_bounds__(kRedCols *kRedStrands) void colreduce_wide_kernel(
+    T *__restrict__ out0, T *__restrict__ out1, T *__restrict__ out2, const float *__restrict__ partial,
+    int blocks_per_sample, int C, int ncols, int col_blocks) {
+    __shared__ float strands[kRedStrands][kRedWideCols + 4];
+    wave_clock_mark(kClockColReduce, 0);
+    const int tx = threadIdx.x % kRedCols;
+    const int ty = threadIdx.x / kRedCols;
+    const int64_t b = blockIdx.x / col_blocks;
+    const int col0 = (int)(blockIdx.x % col_blocks) * kRedWideCols;
+    const int col = col0 + 4 * tx;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (col < ncols) {
+        const float *p = partial + (b * blocks_per_sample) * (int64_t)ncols + col;
+        int g = ty;
+        for (; g + 7 * kRedStrands < blocks_per_sample; g += 8 * kRedStrands) {
+            u32x4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4 *>(p + (int64_t)(g + i * kRedStrands) * ncols);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] += as_f32(v[i][j]);
+        }
+        for (; g < blocks_per_sample; g += kRedStrands) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(p + (int64_t)g * ncols);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] += as_f32(v[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) strands[ty][4 * tx + j] = acc[j];
+    __syncthreads();
+    const int c = col0 + (int)threadIdx.x;
+    if (threadIdx.x < kRedWideCols && c < ncols) {
+        float s = strands[0][threadIdx.x];
+#pragma unroll
+        for (int i = 1; i < kRedStrands; ++i) s += strands[i][threadIdx.x];
+        T *dst = c < C ? out0 : (c < 2 * C ? out1 : out2);  // column sets of C columns each
+        store_scalar<T>(dst + b * C + c % C, s);
+    }
+    wave_clock_mark(kClockColReduce, 1);
+}
+
+// 1: colreduce_wide_kernel where its conditions hold; 0: colreduce_kernel always.  Measured inside cfg3's step with
+// the per-wavefront clocks (256 partial rows of 6144 columns): 3.1 us from first wavefront start to last end for
+// the wide form against 2.3 us for the narrow one, whose 192 workgroups spread the same loads over four times
+// as many wavefronts; the narrow one stays.
+#ifndef TTN_COLREDUCE_WIDE
+#define TTN_COLREDUCE_WIDE 0
+#endif
+
 int launch_colreduce(void *out0, void *out1, void *out2, const float *partial, int64_t batch,
                      int blocks_per_sample, int64_t C, int64_t ncols, int dtype,
                      hipStream_t stream) {
+    if (TTN_COLREDUCE_WIDE && ncols % 4 == 0 && aligned16(partial)) {
+        const int col_blocks = (int)((ncols + kRedWideCols - 1) / kRedWideCols);
+        const int64_t grid = batch * col_blocks;
+        if (grid > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "column reducer grid too large");
+        dim3 g((unsigned)grid), blk(kRedCols * kRedStrands);
+        if (dtype == TT_NORM_BF16)
+            colreduce_wide_kernel<bf16_t><<<g, blk, 0, stream>>>((bf16_t *)out0, (bf16_t *)out1, (bf16_t *)out2, partial,
+                                                                 blocks_per_sample, (int)C, (int)ncols, col_blocks);
+        else if (dtype == TT_NORM_F16)
+            colreduce_wide_kernel<f16_t><<<g, blk, 0, stream>>>((f16_t *)out0, (f16_t *)out1, (f16_t *)out2, partial,
+                                                                blocks_per_sample, (int)C, (int)ncols, col_blocks);
+        else
+            colreduce_wide_kernel<float><<<g, blk, 0, stream>>>((float *)out0, (float *)out1, (float *)out2, partial,
+                                                                blocks_per_sample, (int)C, (int)ncols, col_blocks);
+        return check_launch("column reducer launch");
+    }
     const int col_blocks = (int)((ncols + kRedCols - 1) / kRedCols);
     const int64_t grid = batch * col_blocks;
     if (grid > 0x7fffffffLL) return fail(TT_NORM_EINVAL, "column reducer grid too large");
