@@ -59,6 +59,12 @@ WORKLOADS = {
             "forward and backward of the chain (4 C-ABI calls)",
     "w1536-f16": "237600 tokens x 1536 fp16 (a smaller model's hidden size, the any-width kernels); fused RMSNorm "
                  "fwd+bwd + fused AdaLN fwd+bwd per step (4 C-ABI calls)",
+    "w4096-bf16": "89100 tokens x 4096 bf16 (a wider model's hidden size; rows of 512 16-byte pieces, four wavefronts "
+                  "per row); fused RMSNorm fwd+bwd + fused AdaLN fwd+bwd per step (4 C-ABI calls)",
+    "w5120-bf16": "71280 tokens x 5120 bf16 (640 pieces per row); the same step",
+    "w8192-bf16": "44550 tokens x 8192 bf16 (1024 pieces per row, the widest supported); the same step",
+    "w4096-bf16-gated": "89100 tokens x 4096 bf16; gated residual update fused with the AdaLN that follows it, forward "
+                        "+ backward with a gradient on h2, on the wide-row kernels (2 C-ABI calls)",
     "cfg4-eager-gpu": "cfg4's step computed by the reference's eager formulas as PyTorch ops on the same GPU "
                       "(what the reference runs with FUSED_KERNELS off): a baseline, not this library",
     "qkv-site": "the QK-norm call site through the autograd Function: [1, 29700, 24, 384] bf16 fused projection -> "
@@ -86,6 +92,8 @@ WORKLOADS = {
                      "sets, back to back) seen from inside: every wavefront's start and end on the constant 100 MHz "
                      "clock, from a measurement build of the library (python -m teletron_amd.build --variant LIB "
                      "--flag=-DTTN_WAVE_CLOCK=1, loaded with TELETRON_AMD_LIB=LIB); --steps = timelines collected",
+    "timeline-cfg4": "the same view of cfg4's step (118800 x 3072 bf16, one buffer set): the AdaLN forward and backward "
+                     "kernels and the last column reducer of the step carry the clocks",
     "gated": "118800 tokens x 3072 bf16; gated residual update fused with the AdaLN that follows it, forward "
              "(2 reads, 2 writes) + backward with a gradient on h2 (4 reads, 2 writes) (2 C-ABI calls)",
 }
@@ -140,9 +148,10 @@ def build_workload(name, torch, capi, dev):
         return [("adaln_forward", fwd, 2), ("adaln_backward", bwd, 3)], out
 
     bf = torch.bfloat16
-    if name in ("cfg4", "cfg3", "w1536-f16"):
+    if name in ("cfg4", "cfg3", "w1536-f16", "w4096-bf16", "w5120-bf16", "w8192-bf16"):
         rows, cols, dt = {"cfg4": (ROWS, COLS, bf), "cfg3": (29700, COLS, bf),
-                          "w1536-f16": (2 * ROWS, 1536, torch.float16)}[name]
+                          "w1536-f16": (2 * ROWS, 1536, torch.float16), "w4096-bf16": (89100, 4096, bf),
+                          "w5120-bf16": (71280, 5120, bf), "w8192-bf16": (44550, 8192, bf)}[name]
         x, grad = rnd(rows, cols, dtype=dt), rnd(rows, cols, dtype=dt)
         scale, shift = rnd(1, cols, dtype=dt, k=0.1), rnd(1, cols, dtype=dt, k=0.1)
         calls = []
@@ -273,24 +282,24 @@ def build_workload(name, torch, capi, dev):
 
         fn = fused if name == "qkv-site" else reference_way
         return [(name.replace("-", "_") + "_fwd_bwd", fn, 12)], B * H * S * D * 2, S, "bf16", gq
-    if name == "gated":
-        B, S = 1, ROWS
-        h, a = rnd(B, S, COLS, dtype=bf), rnd(B, S, COLS, dtype=bf)
-        go, g2 = rnd(B, S, COLS, dtype=bf, k=0.1), rnd(B, S, COLS, dtype=bf, k=0.1)
-        gate, scale, shift = (rnd(B, COLS, dtype=bf, k=0.3) for _ in range(3))
+    if name in ("gated", "w4096-bf16-gated"):
+        B, S, W = (1, ROWS, COLS) if name == "gated" else (1, 89100, 4096)
+        h, a = rnd(B, S, W, dtype=bf), rnd(B, S, W, dtype=bf)
+        go, g2 = rnd(B, S, W, dtype=bf, k=0.1), rnd(B, S, W, dtype=bf, k=0.1)
+        gate, scale, shift = (rnd(B, W, dtype=bf, k=0.3) for _ in range(3))
         h2, out, dh, da = (torch.empty_like(h) for _ in range(4))
         mean, rstd = f32(B * S), f32(B * S)
         dq, dsc, dsh = (torch.empty_like(gate) for _ in range(3))
-        n = L.tt_gated_residual_adaln_backward_workspace_bytes(B, S, COLS, capi.BF16)
+        n = L.tt_gated_residual_adaln_backward_workspace_bytes(B, S, W, capi.BF16)
         ws = scratch(n)
         fwd = lambda: ck(L.tt_gated_residual_adaln_forward(p(h2), p(out), p(mean), p(rstd), p(h), p(a), p(gate),
-                                                           p(scale), p(shift), B, S, COLS, EPS, capi.BF16, _LAUNCH_STREAM[0]),
+                                                           p(scale), p(shift), B, S, W, EPS, capi.BF16, _LAUNCH_STREAM[0]),
                          "gated fwd")
         bwd = lambda: ck(L.tt_gated_residual_adaln_backward(p(dh), p(da), p(dq), p(dsc), p(dsh), p(go), p(g2), p(h2),
-                                                            p(a), p(gate), p(scale), p(mean), p(rstd), B, S, COLS,
+                                                            p(a), p(gate), p(scale), p(mean), p(rstd), B, S, W,
                                                             capi.BF16, p(ws), n, _LAUNCH_STREAM[0]), "gated bwd")
         return [("gated_residual_adaln_forward", fwd, 4), ("gated_residual_adaln_backward", bwd, 6)], \
-            S * COLS * 2, S, "bf16", h
+            S * W * 2, S, "bf16", h
     raise ValueError(name)
 
 
@@ -457,8 +466,9 @@ def wave_timeline(args, torch, capi, dev):
         sys.exit(2)
     set_clock.argtypes, set_clock.restype = [ctypes.c_void_p], ctypes.c_int
     clock_bytes.argtypes, clock_bytes.restype = [], ctypes.c_size_t
-    sets = [build_workload("cfg3", torch, capi, dev)[0] for _ in range(3)]
-    rows = 29700
+    base = args.workload[len("timeline-"):]
+    sets = [build_workload(base, torch, capi, dev)[0] for _ in range(3 if base == "cfg3" else 1)]
+    rows = 29700 if base == "cfg3" else ROWS
     buf = torch.zeros(clock_bytes() // 8, dtype=torch.int64, device=dev)
     torch.cuda.synchronize()
     if set_clock(ctypes.c_void_p(buf.data_ptr())) != 0:
@@ -475,7 +485,7 @@ def wave_timeline(args, torch, capi, dev):
             if i == args.warmup:
                 e0.record()
             turn += 1
-            for _, fn, _ in sets[turn % 3]:
+            for _, fn, _ in sets[turn % len(sets)]:
                 fn()
         e1.record()
         torch.cuda.synchronize()
@@ -500,7 +510,9 @@ def wave_timeline(args, torch, capi, dev):
                           "rows_done_first": done.min(), "rows_done_median": float(np.median(done)),
                           "rows_done_last_without_extra": done[~extra].max(),
                           "rows_done_last_with_extra": done[extra].max() if extra.any() else None,
-                          "us_per_row_median": float(np.median((done - st) / (per_wave + extra)))})
+                          "us_per_row_median": float(np.median((done - st) / (per_wave + extra))),
+                          # workgroups are dealt to the eight XCDs in turn
+                          "rows_done_median_by_xcd": [round(float(np.median(done[(w // 4) % 8 == x])), 2) for x in range(8)]})
                 if len(a) % 4 == 0:      # per workgroup: its slowest wavefront's last row -> its partial row written
                     wg_done, wg_end = done.reshape(-1, 4), en.reshape(-1, 4)
                     r["partial_row_flush_median"] = float(np.median(wg_end.max(axis=1) - wg_done.max(axis=1)))
@@ -521,7 +533,7 @@ def wave_timeline(args, torch, capi, dev):
         if vals[0] is None:
             return None
         if isinstance(vals[0], list):
-            return [int(np.median([v[i] for v in vals])) for i in range(len(vals[0]))]
+            return [round(float(np.median([v[i] for v in vals])), 2) for i in range(len(vals[0]))]
         return round(float(np.median(vals)), 2)
 
     out = {}
@@ -529,12 +541,12 @@ def wave_timeline(args, torch, capi, dev):
         out[key] = {k2: med((key, k2)) for k2 in v} if isinstance(v, dict) else med((key,))
     set_clock(None)
     step_us = out["step_us_by_events"]
-    algo = 5 * rows * COLS * 2
+    algo = (5 if base == "cfg3" else 10) * rows * COLS * 2
     print(json.dumps({
-        "metric": "timeline of cfg3's step from per-wavefront clocks (medians, us)", "value": round(algo / step_us / 1e3, 1),
+        "metric": "timeline of %s's step from per-wavefront clocks (medians, us)" % base, "value": round(algo / step_us / 1e3, 1),
         "unit": "GB/s", "n_gpus": 1, "steps": len(collected), "warmup": args.warmup, "ms_per_step": round(step_us / 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": WORKLOADS["timeline-cfg3"], "rows": rows, "cols": COLS}, "timeline_us": out,
+        "config": {"workload": WORKLOADS[args.workload], "rows": rows, "cols": COLS}, "timeline_us": out,
     }))
 
 
@@ -637,7 +649,7 @@ def main():
     if args.workload == "cached-set":
         cached_set(args, torch, capi, dev)
         return
-    if args.workload == "timeline-cfg3":
+    if args.workload.startswith("timeline-"):
         wave_timeline(args, torch, capi, dev)
         return
     calls, tensor_bytes, tokens_per_step, dtype_name, a_tensor = build_workload(args.workload, torch, capi, dev)

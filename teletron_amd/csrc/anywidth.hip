@@ -732,6 +732,7 @@ static int rmsnorm_backward_on(void *dx, void *dw, const void *g, const void *x,
     const size_t need = (size_t)p.blocks * cols * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "rmsnorm backward: workspace %zu B < required %zu B", ws_bytes, need);
+    if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "rmsnorm backward: workspace %p not 16-byte aligned", ws);
     st = dispatch<RmsOn<Map>::template Bwd>(dtype, gc, p, dx, ws, g, x, w, rstd, map, (int)cols, stream);
     if (st != TT_NORM_OK) return st;
     st = check_launch("rmsnorm backward launch");
@@ -819,6 +820,7 @@ static int adaln_backward_any(void *dx, void *dscale, void *dshift, void *dgate,
     const size_t need = (size_t)p.blocks * NSETS * cols * sizeof(float);
     if (!ws || ws_bytes < need)
         return fail(TT_NORM_EWORKSPACE, "adaln backward: workspace %zu B < required %zu B", ws_bytes, need);
+    if (!aligned16(ws)) return fail(TT_NORM_EALIGN, "adaln backward: workspace %p not 16-byte aligned", ws);
     st = dispatch<AdalnOn<GATED, RES>::template Bwd>(dtype, gc, p, dx, ws, g, x, scale, mean, rstd, ex, rows_per_sample,
                                                      layout_of(batch, rows_per_sample, seq_first), (int)cols, stream);
     if (st != TT_NORM_OK) return st;

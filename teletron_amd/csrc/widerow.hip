@@ -1,12 +1,22 @@
 // RMSNorm and AdaLN for WIDE rows: more than 384 16-byte pieces per row (above 3072 two-byte / 1536
-// four-byte columns, up to 1024 pieces).  One wavefront per row would have to hold 8 to 16 accesses
-// per lane and tensor, which leaves a compute unit with too few wavefronts to keep its share of the
-// memory system busy; here the four wavefronts of a workgroup share a row instead: wavefront w owns
-// the contiguous slice of ppw = ceil(pieces / 4) pieces that starts at piece w * ppw (CH = 2, 3 or 4
-// accesses per lane, the last one partly filled when ppw is not a multiple of 64, so the four
-// wavefronts always carry equal shares), the row statistics are exchanged through LDS with one barrier per row, and a lane still owns
-// fixed columns, so the parameter-gradient sums stay in registers and every wavefront writes its own
-// slice of the workgroup's partial row (no cross-wavefront addition at all).
+// four-byte columns, up to 1024 pieces), dense rows only (contiguous, or sample-major / sequence-first AdaLN).
+// One wavefront per row would have to hold 8 to 16 accesses per lane and tensor, which leaves a compute unit
+// with too few wavefronts to keep its share of the memory system busy; here the four wavefronts of a
+// workgroup share a row instead: wavefront w owns the contiguous slice of ppw = ceil(pieces / 4) pieces that
+// starts at piece w * ppw (CH = 2, 3 or 4 accesses per lane, the last one partly filled when ppw is not a
+// multiple of 64, so the four wavefronts always carry equal shares), the row statistics are exchanged through
+// LDS with one barrier per row, and a lane still owns fixed columns, so the parameter-gradient sums stay in
+// registers and every wavefront writes its own slice of the workgroup's partial row (no cross-wavefront
+// addition at all).
+//
+// Grids (measured at 4096, 5120 and 8192 two-byte columns, 730 MB per tensor): RMSNorm forward one-shot (one
+// row per workgroup); AdaLN forward in short-lived workgroups of four rows each, which amortise the set-up of
+// the modulation row (kept as fp32 values) and still retire and get replaced as the grid drains; both request
+// the next row before the current row's output pass.  Backward persistent, two workgroups per compute unit,
+// the next row requested between the two passes, write-through stores.  The gated residual and residual forms
+// (GATED / RES, as in adaln.hip) use the same grids as the plain form, so that the column sums are added in the
+// same order and a fused call is bit-identical to its parts.  Dense fp32 rows of 3072 columns (768 pieces) take
+// their backward here too: a wavefront that owns such a row has registers for one row buffer only.
 //
 // Same arithmetic and rounding points as the kernels in rmsnorm.hip / adaln.hip / anywidth.hip; the
 // variance of AdaLN is formed per wavefront about the wavefront's own mean and merged

@@ -11,6 +11,8 @@ is the command that ran, on committed files only.
     python -m teletron_amd.profile_collect variants  --dir gpurun_out/prof [--only base unpacked ...]
     python -m teletron_amd.profile_collect runs      --dir gpurun_out/prof
     python -m teletron_amd.profile_collect cached    --dir gpurun_out/prof
+    python -m teletron_amd.profile_collect wide      --dir gpurun_out/prof [--only base onewave ...]
+    python -m teletron_amd.profile_collect timeline  --dir gpurun_out/prof
 
 This process never touches the GPU itself (it starts children and nothing else), every child runs under a
 time limit, a failed step ends the collection, and each step prints one line when it starts.
@@ -24,7 +26,8 @@ import sys
 import time
 
 from teletron_amd.build import ROOT
-from teletron_amd.profile_summary import CACHED_VARIANTS, CFG4_PASSES, PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WORKLOAD_INFO
+from teletron_amd.profile_summary import (CACHED_VARIANTS, CFG4_PASSES, PASS_COUNTERS, RUN_LENGTHS, VARIANTS, WIDE_VARIANTS,
+                                          WIDE_WORKLOADS, WORKLOAD_INFO)
 
 BENCH = ["python3", "bench.py"]
 QUICK = ["--steps", "3", "--warmup", "1", "--no-cpu-baseline"]
@@ -137,15 +140,34 @@ def cached(directory, only):
             env={"TELETRON_AMD_LIB": os.path.join(vdir, f"lib_{name}.so")})
 
 
+def wide(directory, only):
+    table = [("wide_" + n, f, w) for n, f, w in WIDE_VARIANTS]
+    vdir = _build_variants(directory, table, ["wide_" + o for o in only] if only else None)
+    for name, flags, _ in WIDE_VARIANTS:
+        if only and name not in only:
+            continue
+        env = {"TELETRON_AMD_LIB": os.path.join(vdir, f"lib_wide_{name}.so")} if flags else None
+        for w in WIDE_WORKLOADS + (["w4096-bf16-gated"] if not flags else []):
+            run([*BENCH, "--steps", "30", "--warmup", "5", "--no-cpu-baseline", "--workload", w],
+                out=os.path.join(directory, f"wide_{name}_{w}.json"), env=env)
+
+
+def timeline(directory, only):
+    vdir = _build_variants(directory, [("waveclock", ["-DTTN_WAVE_CLOCK=1"], "")], None)
+    env = {"TELETRON_AMD_LIB": os.path.join(vdir, "lib_waveclock.so")}
+    run([*BENCH, "--workload", "timeline-cfg3", "--steps", "25", "--warmup", "6"], out=os.path.join(directory, "timeline_cfg3.json"), env=env)
+    run([*BENCH, "--workload", "timeline-cfg4", "--steps", "15", "--warmup", "4"], out=os.path.join(directory, "timeline_cfg4.json"), env=env)
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs", "cached"))
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs", "cached", "wide", "timeline"))
     ap.add_argument("--dir", required=True, help="where the rocprofv3 databases and bench.py lines go")
     ap.add_argument("--only", nargs="*", default=None, help="workloads / variant names to restrict the collection to")
     a = ap.parse_args()
     os.makedirs(a.dir, exist_ok=True)
-    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": runs, "cached": cached}[a.what](
-        a.dir, a.only)
+    {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": runs, "cached": cached,
+     "wide": wide, "timeline": timeline}[a.what](a.dir, a.only)
     print(f"[collect] {a.what}: complete; summarise with `python -m teletron_amd.profile_summary {a.what} --dir {a.dir}`",
           flush=True)
 

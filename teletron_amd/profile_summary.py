@@ -11,6 +11,8 @@ kept under profiles/, plus profiles/cfg4_traffic.json, which bench.py reads for 
     python -m teletron_amd.profile_summary variants --dir rocprof_out      (<dir>/variant_<name>.json, _sq, _stall)
     python -m teletron_amd.profile_summary runs --dir rocprof_out          (<dir>/run_<name>_<workload>.json, run_<name>_trace)
     python -m teletron_amd.profile_summary cached --dir rocprof_out        (<dir>/cached_<name>.json)
+    python -m teletron_amd.profile_summary wide --dir rocprof_out          (<dir>/wide_<variant>_<workload>.json)
+    python -m teletron_amd.profile_summary timeline --dir rocprof_out      (<dir>/timeline_cfg3.json, timeline_cfg4.json)
 
 `python -m teletron_amd.profile_collect <what> --dir <dir>` runs the commands that produce those inputs.
 The databases are large; run this where they were written and keep only what it writes (--out).
@@ -278,6 +280,10 @@ WORKLOAD_INFO = {
     "cfg3": "AdaLN fwd+bwd, 29 700 x 3072 bf16",
     "cfg5": "AdaLN -> RMSNorm chain, 4 x 11 056 x 3072 bf16, one modulation row per sample",
     "w1536-f16": "any-width kernels: RMSNorm + AdaLN fwd+bwd, 237 600 x 1536 fp16",
+    "w4096-bf16": "wide-row kernels (four wavefronts per row): RMSNorm + AdaLN fwd+bwd, 89 100 x 4096 bf16",
+    "w5120-bf16": "wide-row kernels: RMSNorm + AdaLN fwd+bwd, 71 280 x 5120 bf16",
+    "w8192-bf16": "wide-row kernels: RMSNorm + AdaLN fwd+bwd, 44 550 x 8192 bf16",
+    "w4096-bf16-gated": "wide-row kernels: gated residual + AdaLN fwd (2R 2W) + bwd (4R 2W), 89 100 x 4096 bf16",
     "qkv-site": "QK-norm call site through the autograd Function: q and k normalised on the strided views of the "
                 "fused QKV projection, gradients written straight into the projection's gradient",
     "qkv-site-rope": "QK-norm call site with the rotary embedding fused behind the norm",
@@ -418,6 +424,9 @@ VARIANTS = [  # name, hipcc flags of the build ([] = the shipped library), what 
      "before the packed dot-product forms"),
     ("packedproducts", ["-DTTN_BWD_PACKED_MATH=1"],
      "backward: gy / gx = rnd(g * parameter) from packed pairs; the column sums still unpack g"),
+    ("serialflush", ["-DTTN_FLUSH_PARALLEL=0"],
+     "backward: the workgroup's partial row is folded by its four wavefronts in turn (four barriers, 4-byte writes) "
+     "instead of in parallel"),
     ("nodrain", ["-DTTN_BWD_DRAIN_STORES=0"],
      "backward: a row's first pass waits for its own loads only, not for the previous row's stores"),
     ("plainstore", ["-DTTN_RMS_BWD_STORE=0", "-DTTN_ADALN_BWD_STORE=0"],
@@ -649,10 +658,133 @@ backward kernel.  Written by `python -m teletron_amd.profile_summary runs --dir 
     print("wrote qkv_site_run_length_variants.md")
 
 
+WIDE_WORKLOADS = ["w4096-bf16", "w5120-bf16", "w8192-bf16"]
+WIDE_VARIANTS = [  # name, flags, what: the choices of widerow.hip, each measured on the three wide workloads
+    ("base", [], "the shipped kernels"),
+    ("onewave", ["-DTTN_WIDE_ROWS=0"],
+     "one wavefront per row (8, 12 or 16 accesses per lane): the any-width kernels, which strided views still use"),
+    ("rmsfwd_persistent", ["-DTTN_WIDE_RMS_FWD_ROWS_PER_BLOCK=0"], "RMSNorm forward as a persistent grid instead of one-shot"),
+    ("adalnfwd_oneshot", ["-DTTN_WIDE_ADALN_FWD_ROWS_PER_BLOCK=1"], "AdaLN forward one-shot (one row per workgroup)"),
+    ("adalnfwd_persistent", ["-DTTN_WIDE_ADALN_FWD_ROWS_PER_BLOCK=0"], "AdaLN forward as a persistent grid"),
+    ("fwd_noprefetch", ["-DTTN_WIDE_FWD_PREFETCH=0"], "forward: the next row is requested only when the current one is done"),
+    ("adalnfwd_packedparams", ["-DTTN_WIDE_FWD_PARAMS_F32=0"],
+     "AdaLN forward: rnd(1 + scale) and shift stay packed and are unpacked for every row"),
+    ("bwd3", ["-DTTN_WIDE_BWD_BLOCKS_PER_CU=3"], "backward: three workgroups per compute unit instead of two"),
+    ("bwd1", ["-DTTN_WIDE_BWD_BLOCKS_PER_CU=1"], "backward: one workgroup per compute unit"),
+    ("bwd_noprefetch", ["-DTTN_WIDE_BWD_PREFETCH=0"], "backward: no request for the next row between the passes"),
+    ("bwd_plainstore", ["-DTTN_WIDE_BWD_STORE=0"], "backward: plain streaming stores instead of write-through"),
+]
+
+
+def wide(directory):
+    """bench lines wide_<variant>_<workload>.json: the choices of the wide-row kernels on rows of 512, 640 and 1024
+    pieces."""
+    digest = kernel_source_digest()
+    vdir = f"{DIR_SHOWN}/variants"
+    calls = ["rmsnorm_forward", "rmsnorm_backward", "adaln_forward", "adaln_backward"]
+    head = "| variant | " + " | ".join(f"{w}: ms per step, GB/s (% of 8 TB/s); " + " / ".join(c.replace("norm_", " ").replace("ward", "") for c in calls)
+                                        + " µs" for w in WIDE_WORKLOADS) + " |"
+    rows = [head, "|---|" + "---|" * len(WIDE_WORKLOADS)]
+    cmds = []
+    for name, flags, what in WIDE_VARIANTS:
+        cells = []
+        for w in WIDE_WORKLOADS:
+            f = os.path.join(directory, f"wide_{name}_{w}.json")
+            if not os.path.exists(f):
+                cells.append("-")
+                continue
+            b = json.loads(open(f).read().strip().splitlines()[-1])
+            cells.append(f"{b['ms_per_step']:.4f}, {b['value']:.0f} ({100 * b['frac_of_hbm_peak']:.1f}); "
+                         + " / ".join(f"{b['per_call_untimed'][c]['median_us']:.0f}" for c in calls))
+        if all(c == "-" for c in cells):
+            continue
+        rows.append(f"| `{name}` | " + " | ".join(cells) + " |")
+        build = " ".join(f"'--flag={f}'" for f in flags)
+        cmds.append(f"* `{name}`: {what}" + (f"  \n  `python -m teletron_amd.build --variant {vdir}/lib_wide_{name}.so {build}`" if flags else ""))
+    gated = ""
+    g = os.path.join(directory, "wide_base_w4096-bf16-gated.json")
+    if os.path.exists(g):
+        b = json.loads(open(g).read().strip().splitlines()[-1])
+        c = b["per_call_untimed"]
+        gated = (f"\nThe gated residual form on wide rows (`--workload w4096-bf16-gated`, shipped library): {b['ms_per_step']:.4f} ms per "
+                 f"step, {b['value']:.0f} GB/s ({100 * b['frac_of_hbm_peak']:.1f} % of 8 TB/s); forward "
+                 f"{c['gated_residual_adaln_forward']['median_us']:.0f} µs, backward {c['gated_residual_adaln_backward']['median_us']:.0f} µs.\n")
+    md = f"""# Wide rows (more than 384 16-byte pieces): what each choice of widerow.hip is worth
+
+{BOX}.  Kernel sources digest `{digest}`.  Rows of 4096, 5120 and 8192 bf16 columns (512, 640 and 1024 pieces; 730 MB per
+tensor), the cfg4 step (RMSNorm fwd+bwd + AdaLN fwd+bwd, four C-ABI calls) through the unchanged benchmark, each
+variant the shipped sources built with other values of the macros at the top of `widerow.hip`, one box, one after the
+other, by `python -m teletron_amd.profile_collect wide --dir {DIR_SHOWN}`:
+
+    python -m teletron_amd.build --variant {vdir}/lib_wide_<name>.so <flags>
+    TELETRON_AMD_LIB={vdir}/lib_wide_<name>.so  python3 bench.py --steps 30 --warmup 5 --no-cpu-baseline --workload <workload>
+
+{chr(10).join(cmds)}
+
+Per-call figures are HIP-event medians over 30 untimed steps.  Written by
+`python -m teletron_amd.profile_summary wide --dir {DIR_SHOWN}`.
+
+{chr(10).join(rows)}
+{gated}"""
+    with open(os.path.join(PROFILES, "wide_rows_variants.md"), "w") as f:
+        f.write(md)
+    print("wrote wide_rows_variants.md")
+
+
+def timeline(directory):
+    """timeline_<workload>.json (bench.py --workload timeline-cfg3 / timeline-cfg4 through a TTN_WAVE_CLOCK build)."""
+    digest = kernel_source_digest()
+    parts = []
+    for w in ("cfg3", "cfg4"):
+        f = os.path.join(directory, f"timeline_{w}.json")
+        if not os.path.exists(f):
+            continue
+        b = json.loads(open(f).read().strip().splitlines()[-1])
+        t = b["timeline_us"]
+        fw, bw, rd = t["adaln_forward"], t["adaln_backward"], t["column_reducer"]
+        rows = ["| kernel | wavefronts | first start | last start | first end | last end | median wavefront life | "
+                "wavefronts active at 5 %, 15 %, ... 95 % of the kernel's span |", "|---|---|---|---|---|---|---|---|"]
+        for name, k in (("adaln_fwd_kernel", fw), ("adaln_bwd_kernel", bw), ("colreduce_kernel", rd)):
+            rows.append(f"| `{name}` | {k['wavefronts']:.0f} | {k['first_start']:.1f} | {k['last_start']:.1f} | {k['first_end']:.1f} | "
+                        f"{k['last_end']:.1f} | {k['median_wavefront_life']:.1f} | {' '.join(f'{a:.0f}' for a in k['active_at_tenths'])} |")
+        extra = bw.get("rows_done_last_with_extra")
+        parts.append(f"""## {w}: {b['config']['rows']} x {b['config']['cols']} bf16, {b['steps']} timelines, medians, µs from the forward kernel's first wavefront
+
+{chr(10).join(rows)}
+
+* step between two events around it: {t['step_us_by_events']:.1f} µs; first start to the reducer's last end: {t['span']:.1f} µs
+* nothing runs for {t['gap_forward_to_backward']:.1f} µs between the forward kernel's last wavefront and the backward kernel's first,
+  and for {t['gap_backward_to_reducer']:.1f} µs between the backward kernel and the reducer
+* backward: {bw['rows_per_wavefront']:.0f} rows per wavefront ({bw['wavefronts_with_one_more']:.0f} wavefronts carry one more), {bw['us_per_row_median']:.2f} µs per row (median);
+  a wavefront's rows are done at {bw['rows_done_first']:.1f} (first) / {bw['rows_done_median']:.1f} (median) / {bw['rows_done_last_without_extra']:.1f} (last, without an extra row) / {extra if extra is None else format(extra, '.1f')} (last, with one);
+  medians per XCD: {' '.join(f'{x:.1f}' for x in bw['rows_done_median_by_xcd'])}
+* backward: from a workgroup's last row to its partial row written: {bw['partial_row_flush_median']:.2f} µs (median); the four wavefronts of a
+  workgroup finish their rows within {bw['rows_done_spread_inside_workgroup_median']:.2f} µs of each other
+""")
+    md = f"""# A step from the inside: per-wavefront clocks in the AdaLN kernels and the column reducer
+
+{BOX}.  Kernel sources digest `{digest}`.  A measurement build of the library (`-DTTN_WAVE_CLOCK=1`: every wavefront
+of `adaln_fwd_kernel`, `adaln_bwd_kernel` and `colreduce_kernel` stores the constant 100 MHz clock when it starts,
+when its rows are done and when its last memory operation has completed) runs the step back to back; the marks of
+the last step are read back.  By `python -m teletron_amd.profile_collect timeline --dir {DIR_SHOWN}`:
+
+    python -m teletron_amd.build --variant {DIR_SHOWN}/variants/lib_waveclock.so --flag=-DTTN_WAVE_CLOCK=1
+    TELETRON_AMD_LIB={DIR_SHOWN}/variants/lib_waveclock.so  python3 bench.py --workload timeline-cfg3 --steps 25 --warmup 6
+    TELETRON_AMD_LIB={DIR_SHOWN}/variants/lib_waveclock.so  python3 bench.py --workload timeline-cfg4 --steps 15 --warmup 4
+
+Written by `python -m teletron_amd.profile_summary timeline --dir {DIR_SHOWN}`.
+
+{chr(10).join(parts)}
+"""
+    with open(os.path.join(PROFILES, "step_timeline_wave_clocks.md"), "w") as f:
+        f.write(md)
+    print("wrote step_timeline_wave_clocks.md")
+
+
 def main():
     global PROFILES, DIR_SHOWN
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs", "cached"))
+    ap.add_argument("what", choices=("cfg4", "workloads", "stream", "variants", "runs", "cached", "wide", "timeline"))
     ap.add_argument("--dir", default="rocprof_out", help="where rocprofv3 wrote (its -d arguments' parent)")
     ap.add_argument("--out", default=PROFILES, help="where the summaries are written (default: profiles/)")
     a = ap.parse_args()
@@ -660,7 +792,7 @@ def main():
     DIR_SHOWN = a.dir.rstrip("/")
     os.makedirs(PROFILES, exist_ok=True)
     {"cfg4": cfg4, "workloads": workloads, "stream": stream, "variants": variants, "runs": run_lengths,
-     "cached": cached}[a.what](a.dir)
+     "cached": cached, "wide": wide, "timeline": timeline}[a.what](a.dir)
 
 
 if __name__ == "__main__":
