@@ -642,10 +642,14 @@ __device__ __forceinline__ void flush_column_partials(float (&acc)[NSETS][G::CHU
 #pragma unroll
             for (int k = 0; k < CHUNKS; ++k)
 #pragma unroll
-                for (int q = 0; q < VEC / 4; ++q)
-                    mine[(s * C + (k * LANES + l) * VEC) / 4 + q] =
-                        u32x4{as_u32(acc[s][k][4 * q]), as_u32(acc[s][k][4 * q + 1]), as_u32(acc[s][k][4 * q + 2]),
-                              as_u32(acc[s][k][4 * q + 3])};
+                for (int q = 0; q < VEC / 4; ++q) {
+                    // copies the compiler cannot see through: the 16-byte write wants four consecutive registers, and
+                    // without the copies it keeps the accumulators themselves in such groups for the whole kernel,
+                    // which costs the row loop a register move per accumulator and row
+                    float a0 = acc[s][k][4 * q], a1 = acc[s][k][4 * q + 1], a2 = acc[s][k][4 * q + 2], a3 = acc[s][k][4 * q + 3];
+                    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+                    mine[(s * C + (k * LANES + l) * VEC) / 4 + q] = u32x4{as_u32(a0), as_u32(a1), as_u32(a2), as_u32(a3)};
+                }
     }
     __syncthreads();
     const u32x4 *all = reinterpret_cast<const u32x4 *>(lds);

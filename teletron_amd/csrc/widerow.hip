@@ -12,8 +12,8 @@
 // Grids (measured at 4096, 5120 and 8192 two-byte columns, 730 MB per tensor): RMSNorm forward one-shot (one
 // row per workgroup); AdaLN forward in short-lived workgroups of four rows each, which amortise the set-up of
 // the modulation row (kept as fp32 values) and still retire and get replaced as the grid drains; both request
-// the next row before the current row's output pass.  Backward persistent, two workgroups per compute unit,
-// the next row requested between the two passes, write-through stores.  The gated residual and residual forms
+// the next row before the current row's output pass.  Backward persistent, two workgroups per compute unit that
+// overlap each other (no request ahead inside a wavefront), write-through stores.  The gated residual and residual forms
 // (GATED / RES, as in adaln.hip) use the same grids as the plain form, so that the column sums are added in the
 // same order and a fused call is bit-identical to its parts.  Dense fp32 rows of 3072 columns (768 pieces) take
 // their backward here too: a wavefront that owns such a row has registers for one row buffer only.
@@ -57,9 +57,12 @@
 #ifndef TTN_WIDE_FWD_PARAMS_F32
 #define TTN_WIDE_FWD_PARAMS_F32 1
 #endif
-// Backward: 1 = the next row's g and x are requested between the two passes of the current row.
+// Backward: 1 = the next row's g and x are requested between the two passes of the current row; 0 = a row is
+// requested when the one before it is done (the two workgroups of a compute unit overlap each other instead:
+// 347 / 372 us against 380 / 385 us for RMSNorm / AdaLN backward at 89 100 x 4096 two-byte columns, and one
+// workgroup per compute unit without the request ahead is far slower, 504 / 560 us).
 #ifndef TTN_WIDE_BWD_PREFETCH
-#define TTN_WIDE_BWD_PREFETCH 1
+#define TTN_WIDE_BWD_PREFETCH 0
 #endif
 
 namespace ttn {
@@ -67,8 +70,12 @@ namespace ttn {
 #ifndef TTN_GATED_3072_WIDE
 #define TTN_GATED_3072_WIDE 0
 #endif
+// Measurement builds: 1 = the dense backward at 3072 two-byte columns on these kernels instead of the tuned ones.
+#ifndef TTN_16BIT_3072_BWD_WIDE
+#define TTN_16BIT_3072_BWD_WIDE 0
+#endif
 // narrower rows belong to the one-wavefront-per-row kernels
-constexpr int kWidePiecesMin = TTN_GATED_3072_WIDE ? 384 : 385;
+constexpr int kWidePiecesMin = (TTN_GATED_3072_WIDE || TTN_16BIT_3072_BWD_WIDE) ? 384 : 385;
 
 // Which of this lane's CH accesses lie inside a row of `pieces` 16-byte pieces, for wavefront `wave`.
 template <int CH>
@@ -261,9 +268,13 @@ __device__ __forceinline__ void wide_store_partials(float (&acc)[NSETS][CH][Elem
             if (!m.in[k]) continue;
             float *p = partial_row + (int64_t)s * C + slice + (k * kWaveSize + lane) * VEC;
 #pragma unroll
-            for (int q = 0; q < VEC / 4; ++q)
-                *reinterpret_cast<u32x4 *>(p + 4 * q) = u32x4{as_u32(acc[s][k][4 * q]), as_u32(acc[s][k][4 * q + 1]),
-                                                              as_u32(acc[s][k][4 * q + 2]), as_u32(acc[s][k][4 * q + 3])};
+            for (int q = 0; q < VEC / 4; ++q) {
+                // copies the compiler cannot see through, so that the 16-byte store does not pin the accumulators to
+                // groups of four consecutive registers for the whole kernel (see flush_column_partials)
+                float a0 = acc[s][k][4 * q], a1 = acc[s][k][4 * q + 1], a2 = acc[s][k][4 * q + 2], a3 = acc[s][k][4 * q + 3];
+                asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+                *reinterpret_cast<u32x4 *>(p + 4 * q) = u32x4{as_u32(a0), as_u32(a1), as_u32(a2), as_u32(a3)};
+            }
         }
 }
 
@@ -750,6 +761,7 @@ bool gated_forward_on_wide_rows(int64_t cols, int dtype) {
     return TTN_GATED_3072_WIDE && TTN_WIDE_ROWS && dtype != TT_NORM_F32 && cols == 3072;
 }
 bool dense_backward_on_wide_rows(int64_t cols, int dtype) {
+    if (TTN_16BIT_3072_BWD_WIDE && TTN_WIDE_ROWS && dtype != TT_NORM_F32 && cols == 3072) return true;
     return TTN_F32_3072_BWD_WIDE && TTN_WIDE_ROWS && dtype == TT_NORM_F32 && cols == 3072;
 }
 

@@ -440,8 +440,9 @@ VARIANTS = [  # name, hipcc flags of the build ([] = the shipped library), what 
      "backward: two workgroups per compute unit (two wavefronts per SIMD, half the registers each)"),
     ("loadcached", ["-DTTN_BWD_LOAD_POLICY=0"],
      "backward: row loads without the non-temporal hint (buffer loads, default cache policy)"),
-    ("loadsystem", ["-DTTN_BWD_LOAD_POLICY=19"],
-     "backward: row loads marked sc0 sc1 nt (system scope + non-temporal)"),
+    ("loadplain", ["-DTTN_BWD_LOAD_POLICY=-1"],
+     "backward: plain global loads with the non-temporal hint instead of buffer loads marked sc0 sc1 nt (system scope + "
+     "non-temporal)"),
     ("grid88", ["-DTTN_BWD_GRID_PERCENT=88"],
      "backward: persistent grid over 88 % of the compute units (226 workgroups instead of 256)"),
     ("fwd5", ["-DTTN_RMS_FWD_DYN_LDS=(C>=1024?(sizeof(T)==2?0:76800):0)"],
@@ -514,9 +515,13 @@ and the kernels' duration does not follow: the time goes to waiting instead (SQ_
 SQ_ACTIVE_INST_ANY loses).  The backward kernels are not limited by instruction issue.  Memory pipeline: every
 alternative keeps more requests in flight per wavefront than the shipped pipeline (or, for `onebuffer`, fewer) and
 is slower; the slower ones show more DRAM-credit stall cycles at the L2-to-memory interface, i.e. the extra
-requests queue instead of being served.  Loads without the non-temporal hint cost 10 %; no other cache policy
-of the loads, and no smaller grid, gains anything.  None reaches the 80 % line; see stream_ceiling.md for what
-plain streams of the same read/write mix reach.
+requests queue instead of being served.  Row loads: without the non-temporal hint (`loadcached`) the backward kernels
+lose 10 %; marked system scope + non-temporal (shipped) they gain about half a per cent over plain non-temporal
+global loads (`loadplain`), the only cache policy that gained anything.  A smaller grid gains nothing.  `serialflush`
+is the end of the kernel only (a workgroup's partial row written after four barriers instead of one: 4.0 us
+against 1.4 us per workgroup by the wave clocks of step_timeline_wave_clocks.md), below what this table
+resolves at 118 800 rows.  None reaches the 80 % line; see stream_ceiling.md for what plain streams of the
+same read/write mix reach.
 """
     with open(os.path.join(PROFILES, "bench_cfg4_tuning_variants.md"), "w") as f:
         f.write(md)
@@ -671,7 +676,9 @@ WIDE_VARIANTS = [  # name, flags, what: the choices of widerow.hip, each measure
      "AdaLN forward: rnd(1 + scale) and shift stay packed and are unpacked for every row"),
     ("bwd3", ["-DTTN_WIDE_BWD_BLOCKS_PER_CU=3"], "backward: three workgroups per compute unit instead of two"),
     ("bwd1", ["-DTTN_WIDE_BWD_BLOCKS_PER_CU=1"], "backward: one workgroup per compute unit"),
-    ("bwd_noprefetch", ["-DTTN_WIDE_BWD_PREFETCH=0"], "backward: no request for the next row between the passes"),
+    ("bwd_prefetch", ["-DTTN_WIDE_BWD_PREFETCH=1"], "backward: the next row is requested between the two passes of the current one"),
+    ("bwd1_prefetch", ["-DTTN_WIDE_BWD_PREFETCH=1", "-DTTN_WIDE_BWD_BLOCKS_PER_CU=1"],
+     "backward: one workgroup per compute unit with the next row requested between the passes"),
     ("bwd_plainstore", ["-DTTN_WIDE_BWD_STORE=0"], "backward: plain streaming stores instead of write-through"),
 ]
 

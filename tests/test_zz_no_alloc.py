@@ -13,6 +13,9 @@ pytestmark = pytest.mark.gpu
 EPS = 1e-6
 
 
+_CALLED_BEFORE = {}
+
+
 def _p(t):
     return ctypes.c_void_p(t.data_ptr())
 
@@ -28,10 +31,17 @@ def _both_ways(capi, device, batch, rows_per_sample, cols, dtype, seed):
     dx = torch.full_like(x, 7.0)
     ds, dh = torch.full_like(scale, 7.0), torch.full_like(scale, 7.0)
     stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(device)[0]      # hipMemGetInfo: device memory not held by any allocation
     st = L.tt_adaln_backward_static(_p(dx), _p(ds), _p(dh), _p(grad), _p(x), _p(scale), _p(mean), _p(rstd),
                                     batch, rows_per_sample, cols, code, stream)
     assert st == 0, (st, L.tt_norm_last_error())
     torch.cuda.synchronize()
+    # the first call on a device may load the library's code object (and with it the static array); later calls
+    # must leave the device's free memory exactly where it was
+    if _CALLED_BEFORE.get(str(device)):
+        assert torch.cuda.mem_get_info(device)[0] == free_before, "tt_adaln_backward_static changed the free device memory"
+    _CALLED_BEFORE[str(device)] = True
     what = f"batch={batch} rows_per_sample={rows_per_sample} cols={cols} {dtype}"
     assert torch.equal(dx, want_dx), "dx " + what
     assert torch.equal(ds, want_ds), "dscale " + what
