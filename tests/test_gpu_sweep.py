@@ -54,9 +54,18 @@ def test_random_rmsnorm_dense_and_strided(capi, gpu_device, cols, dtype, rows, b
         xv = view.transpose(0, 1)                                  # [heads, seq, cols], strided
         assert not xv.is_contiguous()
         out_s, rstd_s = capi.rmsnorm_forward_strided(xv, w, EPS)
-        assert torch.equal(out_s.reshape(rows, cols), out) and torch.equal(rstd_s, rstd)
         dx_s, dw_s = capi.rmsnorm_backward_strided(g.reshape(heads, seq, cols), xv, w, rstd_s)
-        assert torch.equal(dx_s.contiguous().reshape(rows, cols), dx)
+        out_s, dx_s = out_s.reshape(rows, cols), dx_s.contiguous().reshape(rows, cols)
+        if cols * x.element_size() // 16 <= 384:
+            assert torch.equal(out_s, out) and torch.equal(rstd_s, rstd) and torch.equal(dx_s, dx)
+        else:
+            # dense rows of more than 384 pieces run on other kernels (four wavefronts per row) than a strided view of
+            # them: the row sums are formed in another order, so the two agree to fp32 rounding, not bit for bit
+            torch.testing.assert_close(rstd_s, rstd, rtol=1e-6, atol=0)
+            tol = dict(rtol=1e-5, atol=1e-6) if dtype == F32 else dict(rtol=2.0 ** -7, atol=1e-6)
+            torch.testing.assert_close(out_s.float(), out.float(), **tol)
+            torch.testing.assert_close(dx_s.float(), dx.float(), **tol)
+            assert (out_s != out).float().mean() <= 1e-3 and (dx_s != dx).float().mean() <= 1e-2
         colsum_ok(dw_s, want_dw, d["grad"].float() * want_out.float(), 0, "dweight (strided)")
 
 
