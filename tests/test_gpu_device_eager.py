@@ -89,7 +89,9 @@ def _stress_rows(B, S, C, dtype, kind, seed):
 
 
 @pytest.mark.parametrize("C,dtype", [(3072, torch.bfloat16), (1536, torch.bfloat16), (256, torch.bfloat16),
-                                     (64, torch.bfloat16), (3072, torch.float16)])
+                                     (64, torch.bfloat16), (3072, torch.float16),
+                                     # rows shared by four wavefronts (per-wavefront variance about its own mean, merged)
+                                     (4096, torch.bfloat16), (5128, torch.bfloat16), (8192, torch.float16)])
 @pytest.mark.parametrize("kind", ["mean", "outliers"])
 def test_adaln_stress_rows_against_device_eager(capi, gpu_device, C, dtype, kind):
     B, S = 2, 515
