@@ -24,6 +24,9 @@ ADALN_CASES = [
     (2, 130, 1024, HF), (3, 77, 1536, BF), (2, 300, 2048, BF), (5, 33, 3072, HF), (2, 65, 4096, BF),
     (2, 130, 5120, BF), (3, 40, 6144, BF), (2, 35, 6144, HF), (2, 66, 8192, BF), (1, 9, 8192, HF),
     (2, 50, 64, F32), (3, 100, 1000, F32), (2, 40, 4096, F32),
+    # wide rows with more samples than the persistent grid has workgroups (one workgroup per sample), with fewer rows
+    # per sample than a sample's share of the grid, and a single row
+    (700, 3, 4096, BF), (3, 2, 8192, BF), (1, 1, 5120, HF), (600, 1, 2048, F32),
 ]
 
 
