@@ -5,14 +5,14 @@ one block for more counters than it has hangs).  Tuning variants are built here 
 `python -m teletron_amd.build --variant <dir>/variants/lib_<name>.so`, so every command a summary prints
 is the command that ran, on committed files only.
 
-    python -m teletron_amd.profile_collect cfg4      --dir gpurun_out/prof
-    python -m teletron_amd.profile_collect workloads --dir gpurun_out/prof [--only cfg1 cfg3 ...]
-    python -m teletron_amd.profile_collect stream    --dir gpurun_out/prof
-    python -m teletron_amd.profile_collect variants  --dir gpurun_out/prof [--only base unpacked ...]
-    python -m teletron_amd.profile_collect runs      --dir gpurun_out/prof
-    python -m teletron_amd.profile_collect cached    --dir gpurun_out/prof
-    python -m teletron_amd.profile_collect wide      --dir gpurun_out/prof [--only base onewave ...]
-    python -m teletron_amd.profile_collect timeline  --dir gpurun_out/prof
+    python -m teletron_amd.profile_collect cfg4      --dir rocprof_out
+    python -m teletron_amd.profile_collect workloads --dir rocprof_out [--only cfg1 cfg3 ...]
+    python -m teletron_amd.profile_collect stream    --dir rocprof_out
+    python -m teletron_amd.profile_collect variants  --dir rocprof_out [--only base unpacked ...]
+    python -m teletron_amd.profile_collect runs      --dir rocprof_out
+    python -m teletron_amd.profile_collect cached    --dir rocprof_out
+    python -m teletron_amd.profile_collect wide      --dir rocprof_out [--only base onewave ...]
+    python -m teletron_amd.profile_collect timeline  --dir rocprof_out
 
 This process never touches the GPU itself (it starts children and nothing else), every child runs under a
 time limit, a failed step ends the collection, and each step prints one line when it starts.
